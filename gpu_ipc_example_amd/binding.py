@@ -1,0 +1,280 @@
+"""ctypes binding of libvrank_allreduce.so (the C ABI in include/vrank_allreduce.h).
+
+No fallback exists: if the shared library is missing or a call fails, an
+exception is raised.  Device buffers are plain integers (device addresses), so
+callers may hand in ``torch.Tensor.data_ptr()`` values or use the library's own
+vr_malloc plumbing through :class:`DeviceBuffer`.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libvrank_allreduce.so")
+
+ALGOS = ("small", "simple", "bisect", "parallel", "small_pcie_p", "simple_pcie_p", "small_ring",
+         "simple_ring", "small_pcie", "simple_pcie", "allgather_small", "allgather_simple")
+TRANSPORT_DEFAULT, TRANSPORT_DIRECT, TRANSPORT_WIRE = 0, 1, 2
+
+# vr_status -> Python exception class; the texts come from vr_strerror.
+STATUS_NAMES = {
+    1: "UNALIGNED", 2: "UNEVEN", 3: "ALGO", 4: "TOPOLOGY", 5: "SUBGROUP", 6: "GEOMETRY",
+    7: "INVALID", 8: "HIP", 9: "NO_DEVICE", 10: "TIMEOUT", 11: "OVERLAP",
+}
+
+
+class VRError(RuntimeError):
+    def __init__(self, status, message, detail):
+        super().__init__("%s (%s)" % (message, detail) if detail else message)
+        self.status = status
+        self.code = STATUS_NAMES.get(status, str(status))
+        self.message = message
+        self.detail = detail
+
+
+class Geometry(C.Structure):
+    _fields_ = [("groups", C.c_uint32), ("subgroups", C.c_uint32), ("steps", C.c_uint32)]
+
+
+def library_path():
+    return _SO
+
+
+def build_library(force=False):
+    """Compile the gfx950 library in-tree with hipcc (works without a GPU)."""
+    args = ["make", "-s", "-C", os.path.join(_HERE, "csrc"), "-j8"]
+    if force:
+        subprocess.run(args + ["clean"], check=True)
+    subprocess.run(args, check=True)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        raise ImportError(
+            "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `make -C gpu_ipc_example_amd/csrc`" % _SO)
+    L = C.CDLL(_SO)
+    vp, vpp, sz, u32, i = C.c_void_p, C.POINTER(C.c_void_p), C.c_size_t, C.c_uint32, C.c_int
+    sig = {
+        "vr_ctx_create": (i, [i, i, vpp]),
+        "vr_ctx_destroy": (i, [vp]),
+        "vr_ctx_nranks": (i, [vp]),
+        "vr_algo_from_string": (i, [C.c_char_p, C.POINTER(i)]),
+        "vr_algo_name": (C.c_char_p, [i]),
+        "vr_algo_is_allgather": (i, [i]),
+        "vr_algo_message_bytes": (sz, [i]),
+        "vr_check_allreduce": (i, [i, i, vpp, sz, C.POINTER(sz)]),
+        "vr_check_allgather": (i, [i, i, vpp, vpp, sz, C.POINTER(sz)]),
+        "vr_launch_geometry": (i, [i, i, sz, C.POINTER(Geometry)]),
+        "vr_allreduce": (i, [vp, vp, i, i, vpp, vpp, sz, C.POINTER(u32)]),
+        "vr_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, C.POINTER(u32)]),
+        "vr_allreduce_grid": (i, [vp, vp, i, i, vpp, vpp, sz, u32, u32, u32, u32]),
+        "vr_ctx_check": (i, [vp, vp]),
+        "vr_ctx_set_spin_limit": (i, [vp, C.c_uint64]),
+        "vr_ctx_set_tuning": (i, [vp, C.c_char_p, i]),
+        "vr_ctx_get_tuning": (i, [vp, C.c_char_p, C.POINTER(i)]),
+        "vr_time_allreduce": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
+        "vr_time_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
+        "vr_time_copy": (i, [vp, vp, vp, vp, sz, i, C.POINTER(C.c_float)]),
+        "vr_fill_pattern": (None, [C.POINTER(C.c_uint16), i, sz]),
+        "vr_generate": (None, [C.POINTER(C.c_uint16), sz, C.c_uint64, i, C.c_double, C.c_double]),
+        "vr_parse_nelems": (i, [C.c_char_p, C.POINTER(sz)]),
+        "vr_device_count": (i, [C.POINTER(i)]),
+        "vr_device_name": (i, [i, C.c_char_p, sz]),
+        "vr_malloc": (i, [i, sz, vpp]),
+        "vr_free": (i, [vp]),
+        "vr_memset": (i, [vp, i, sz]),
+        "vr_copy_to_device": (i, [vp, vp, sz]),
+        "vr_copy_to_host": (i, [vp, vp, sz]),
+        "vr_stream_create": (i, [i, vpp]),
+        "vr_stream_destroy": (i, [vp]),
+        "vr_stream_sync": (i, [vp]),
+        "vr_strerror": (C.c_char_p, [i]),
+        "vr_last_error_detail": (C.c_char_p, []),
+        "vr_version": (C.c_char_p, []),
+    }
+    for name, (res, args) in sig.items():
+        f = getattr(L, name)          # AttributeError here = header and library disagree
+        f.restype, f.argtypes = res, args
+    L._signatures = sig
+    _lib = L
+    return L
+
+
+def _check(status):
+    if status != 0:
+        L = lib()
+        raise VRError(status, L.vr_strerror(status).decode(), L.vr_last_error_detail().decode())
+
+
+def algo_id(name):
+    out = C.c_int(-1)
+    _check(lib().vr_algo_from_string(name.encode(), C.byref(out)))
+    return out.value
+
+
+def parse_nelems(text):
+    out = C.c_size_t(0)
+    _check(lib().vr_parse_nelems(text.encode(), C.byref(out)))
+    return out.value
+
+
+def _table(ptrs):
+    return (C.c_void_p * len(ptrs))(*[C.c_void_p(int(p)) for p in ptrs])
+
+
+def check_allreduce(algo, nranks, ptrs, nelems):
+    work = C.c_size_t(0)
+    _check(lib().vr_check_allreduce(algo_id(algo), nranks, _table(ptrs), nelems, C.byref(work)))
+    return work.value
+
+
+def launch_geometry(algo, nranks, nelems):
+    g = Geometry()
+    _check(lib().vr_launch_geometry(algo_id(algo), nranks, nelems, C.byref(g)))
+    return g.groups, g.subgroups, g.steps
+
+
+def fill_pattern(rank, n):
+    a = np.empty(n, np.uint16)
+    lib().vr_fill_pattern(a.ctypes.data_as(C.POINTER(C.c_uint16)), rank, n)
+    return a
+
+
+def generate(n, seed, dist, p0, p1):
+    a = np.empty(n, np.uint16)
+    lib().vr_generate(a.ctypes.data_as(C.POINTER(C.c_uint16)), n, seed, dist, p0, p1)
+    return a
+
+
+def device_count():
+    n = C.c_int(0)
+    _check(lib().vr_device_count(C.byref(n)))
+    return n.value
+
+
+def device_name(device=0):
+    buf = C.create_string_buffer(256)
+    _check(lib().vr_device_name(device, buf, 256))
+    return buf.value.decode()
+
+
+class DeviceBuffer:
+    """A vr_malloc'ed region; `.ptr` is the device address."""
+
+    def __init__(self, nbytes, device=0):
+        p = C.c_void_p()
+        _check(lib().vr_malloc(device, nbytes, C.byref(p)))
+        self.ptr, self.nbytes = p.value, nbytes
+
+    def upload(self, arr, offset=0):
+        arr = np.ascontiguousarray(arr)
+        assert offset + arr.nbytes <= self.nbytes
+        _check(lib().vr_copy_to_device(C.c_void_p(self.ptr + offset), arr.ctypes.data_as(C.c_void_p),
+                                       arr.nbytes))
+
+    def download(self, dtype=np.uint16, count=None, offset=0):
+        item = np.dtype(dtype).itemsize
+        if count is None:
+            count = (self.nbytes - offset) // item
+        out = np.empty(count, dtype)
+        _check(lib().vr_copy_to_host(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr + offset),
+                                     out.nbytes))
+        return out
+
+    def fill(self, byte):
+        _check(lib().vr_memset(C.c_void_p(self.ptr), byte, self.nbytes))
+
+    def free(self):
+        if self.ptr:
+            _check(lib().vr_free(C.c_void_p(self.ptr)))
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class VirtualRanks:
+    """N virtual ranks on one GPU: the handle every collective call goes through."""
+
+    def __init__(self, nranks, device=0):
+        h = C.c_void_p()
+        _check(lib().vr_ctx_create(device, nranks, C.byref(h)))
+        self._h, self.nranks, self.device = h, nranks, device
+        self.seq_no = C.c_uint32(1)
+
+    def close(self):
+        if self._h:
+            lib().vr_ctx_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_tuning(self, **kw):
+        for k, v in kw.items():
+            _check(lib().vr_ctx_set_tuning(self._h, k.encode(), int(v)))
+
+    def get_tuning(self, key):
+        v = C.c_int(0)
+        _check(lib().vr_ctx_get_tuning(self._h, key.encode(), C.byref(v)))
+        return v.value
+
+    def set_spin_limit(self, polls):
+        _check(lib().vr_ctx_set_spin_limit(self._h, polls))
+
+    def allreduce(self, algo, bufs, nelems, outs=None, transport=TRANSPORT_DEFAULT, stream=None):
+        assert len(bufs) == self.nranks
+        _check(lib().vr_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
+                                  _table(outs) if outs is not None else None, nelems,
+                                  C.byref(self.seq_no)))
+
+    def allreduce_grid(self, algo, bufs, nelems, groups, subgroups, simd=16, outs=None,
+                       transport=TRANSPORT_DEFAULT, stream=None, seq_no=0xE00F100F):
+        _check(lib().vr_allreduce_grid(self._h, stream, algo_id(algo), transport, _table(bufs),
+                                       _table(outs) if outs is not None else None, nelems, seq_no,
+                                       groups, subgroups, simd))
+
+    def allgather(self, algo, inputs, outputs, nelems, transport=TRANSPORT_DEFAULT, stream=None):
+        _check(lib().vr_allgather(self._h, stream, algo_id(algo), transport, _table(inputs),
+                                  _table(outputs), nelems, C.byref(self.seq_no)))
+
+    def check(self, stream=None):
+        _check(lib().vr_ctx_check(self._h, stream))
+
+    def sync(self, stream=None):
+        _check(lib().vr_stream_sync(stream))
+
+    def time_allreduce(self, algo, bufs, nelems, iters, outs=None, transport=TRANSPORT_DEFAULT,
+                       stream=None):
+        ms = (C.c_float * iters)()
+        _check(lib().vr_time_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
+                                       _table(outs) if outs is not None else None, nelems, iters, ms))
+        return np.frombuffer(ms, np.float32).copy()
+
+    def time_allgather(self, algo, inputs, outputs, nelems, iters, transport=TRANSPORT_DEFAULT,
+                       stream=None):
+        ms = (C.c_float * iters)()
+        _check(lib().vr_time_allgather(self._h, stream, algo_id(algo), transport, _table(inputs),
+                                       _table(outputs), nelems, iters, ms))
+        return np.frombuffer(ms, np.float32).copy()
+
+    def time_copy(self, dst, src, nbytes, iters, stream=None):
+        ms = (C.c_float * iters)()
+        _check(lib().vr_time_copy(self._h, stream, C.c_void_p(int(dst)), C.c_void_p(int(src)), nbytes,
+                                  iters, ms))
+        return np.frombuffer(ms, np.float32).copy()

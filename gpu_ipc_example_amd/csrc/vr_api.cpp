@@ -1,0 +1,661 @@
+// C ABI of the virtual-rank all-reduce library: validation, dispatch, timing and
+// small host utilities.  Device work lives in vr_direct.hip / vr_wire.hip.
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+#include "vr_internal.h"
+
+using namespace vr;
+
+// ---------------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------------
+
+static thread_local std::string g_detail;
+
+static int fail(int status, const std::string &detail) {
+  g_detail = detail;
+  return status;
+}
+
+static int fail_hip(hipError_t e, const char *what) {
+  return fail(VR_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                             \
+  do {                                            \
+    hipError_t e__ = (expr);                      \
+    if (e__ != hipSuccess) return fail_hip(e__, #expr); \
+  } while (0)
+
+extern "C" const char *vr_strerror(int status) {
+  switch (status) {
+    case VR_OK: return "ok";
+    case VR_ERR_UNALIGNED: return "We only support aligned pointer for now";
+    case VR_ERR_UNEVEN: return "We don't support non-even divide yet";
+    case VR_ERR_ALGO: return "Transmit type not support";
+    case VR_ERR_TOPOLOGY: return "Unsupported communication topology";
+    case VR_ERR_SUBGROUP: return "Unsupported Sub-group size";
+    case VR_ERR_GEOMETRY: return "Subgroup numbers must be multiple of 4";
+    case VR_ERR_INVALID: return "invalid argument";
+    case VR_ERR_HIP: return "HIP runtime error";
+    case VR_ERR_NO_DEVICE: return "no gfx950 device";
+    case VR_ERR_TIMEOUT: return "flag poll exceeded its spin limit";
+    case VR_ERR_OVERLAP: return "output partially overlaps an input";
+    default: return "unknown status";
+  }
+}
+
+extern "C" const char *vr_last_error_detail(void) { return g_detail.c_str(); }
+extern "C" const char *vr_version(void) { return "vrank_allreduce 0.1 (gfx950)"; }
+
+// ---------------------------------------------------------------------------------
+// algorithm table
+// ---------------------------------------------------------------------------------
+
+enum TransmitKind { T_PARALLEL, T_BISECT, T_RING, T_SEQUENTIAL };
+
+struct AlgoInfo {
+  const char *name;
+  TransmitKind transmit;
+  int msg_bytes;       // sizeof(message_t) at sub-group size 16
+  int wire_capacity;   // payload bytes per wire at sub-group size 16
+  bool allgather;
+  Order order;
+  bool latency_tuned;  // "small" family: one-shot grid, cached accesses
+};
+
+// message_t / wireCapacity: rt64.hpp:335-340 (8 B, 64 B), rt64_128.hpp:539-551 (8 B, 120 B),
+// rt64.hpp:3-20 (16 B, 128 B), rt64_128.hpp:3-30 (16 B, 240 B), bisect_transmit.hpp:17-25.
+static const AlgoInfo kAlgos[VR_ALGO_COUNT_] = {
+    {"small", T_PARALLEL, 8, 64, false, ORDER_ROTATED, true},
+    {"simple", T_PARALLEL, 8, 120, false, ORDER_ROTATED, false},
+    {"bisect", T_BISECT, 8, 120, false, ORDER_BISECT, false},
+    {"parallel", T_PARALLEL, 8, 120, false, ORDER_ROTATED, false},
+    {"small_pcie_p", T_PARALLEL, 16, 128, false, ORDER_ROTATED, true},
+    {"simple_pcie_p", T_PARALLEL, 16, 240, false, ORDER_ROTATED, false},
+    {"small_ring", T_RING, 16, 128, false, ORDER_ROTATED, true},
+    {"simple_ring", T_RING, 16, 240, false, ORDER_ROTATED, false},
+    {"small_pcie", T_SEQUENTIAL, 16, 128, false, ORDER_ROTATED, true},
+    {"simple_pcie", T_SEQUENTIAL, 16, 240, false, ORDER_ROTATED, false},
+    {"allgather_small", T_RING, 16, 128, true, ORDER_ROTATED, true},
+    {"allgather_simple", T_RING, 16, 240, true, ORDER_ROTATED, false},
+};
+
+static const AlgoInfo *algo_info(int algo) {
+  return (algo >= 0 && algo < VR_ALGO_COUNT_) ? &kAlgos[algo] : nullptr;
+}
+
+extern "C" int vr_algo_from_string(const char *name, int *algo_out) {
+  if (!name) return fail(VR_ERR_INVALID, "null algo name");
+  for (int i = 0; i < VR_ALGO_COUNT_; ++i)
+    if (strcmp(name, kAlgos[i].name) == 0) {
+      if (algo_out) *algo_out = i;
+      return VR_OK;
+    }
+  return fail(VR_ERR_ALGO, std::string("unknown algo '") + name + "'");
+}
+
+extern "C" const char *vr_algo_name(int algo) {
+  const AlgoInfo *a = algo_info(algo);
+  return a ? a->name : "?";
+}
+
+extern "C" int vr_algo_is_allgather(int algo) {
+  const AlgoInfo *a = algo_info(algo);
+  return a ? (a->allgather ? 1 : 0) : 0;
+}
+
+extern "C" size_t vr_algo_message_bytes(int algo) {
+  const AlgoInfo *a = algo_info(algo);
+  return a ? (size_t)a->msg_bytes : 0;
+}
+
+// World sizes each dispatcher switches over (allreduce.cpp:854-881, 1003-1030).
+static int check_topology(const AlgoInfo *a, int nranks) {
+  const bool ok = (a->transmit == T_BISECT) ? (nranks == 4 || nranks == 8 || nranks == 16)
+                                            : (nranks == 2 || nranks == 4 || nranks == 8);
+  if (!ok) return fail(VR_ERR_TOPOLOGY, std::string(a->name) + " does not run on " + std::to_string(nranks) + " ranks");
+  return VR_OK;
+}
+
+static inline size_t div_up(size_t x, size_t m) { return (x + m - 1) / m; }
+
+// calcWorkSize (allreduce.hpp:108-122): alignment is tested before divisibility.
+static int calc_work_size(uintptr_t addr, size_t bytes, size_t nchunks, size_t msg, size_t *work) {
+  if (addr % msg != 0) return VR_ERR_UNALIGNED;
+  const size_t msgs = div_up(bytes, msg);
+  const size_t chunk = div_up(msgs, nchunks);
+  if (msgs * msg != bytes || chunk * msg * nchunks > bytes) return VR_ERR_UNEVEN;
+  *work = chunk * msg;
+  return VR_OK;
+}
+
+extern "C" int vr_check_allreduce(int algo, int nranks, const void *const bufs[], size_t nelems,
+                                  size_t *work_bytes) {
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
+  if (!bufs) return fail(VR_ERR_INVALID, "null buffer table");
+  if (int rc = check_topology(a, nranks)) return rc;
+  size_t work = 0;
+  for (int r = 0; r < nranks; ++r) {
+    if (!bufs[r] && nelems) return fail(VR_ERR_INVALID, "null buffer for rank " + std::to_string(r));
+    int rc = calc_work_size((uintptr_t)bufs[r], nelems * 2, (size_t)nranks, (size_t)a->msg_bytes, &work);
+    if (rc) return fail(rc, "rank " + std::to_string(r) + ", nelems " + std::to_string(nelems));
+  }
+  if (work_bytes) *work_bytes = work;
+  return VR_OK;
+}
+
+extern "C" int vr_check_allgather(int algo, int nranks, const void *const inputs[],
+                                  void *const outputs[], size_t nelems, size_t *work_bytes) {
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
+  if (!inputs || !outputs) return fail(VR_ERR_INVALID, "null buffer table");
+  if (int rc = check_topology(a, nranks)) return rc;
+  size_t work = 0;
+  for (int r = 0; r < nranks; ++r) {
+    if ((!inputs[r] || !outputs[r]) && nelems) return fail(VR_ERR_INVALID, "null buffer for rank " + std::to_string(r));
+    // allgather.hpp:104-117: input and output alignment, then whole messages.
+    if ((uintptr_t)inputs[r] % a->msg_bytes || (uintptr_t)outputs[r] % a->msg_bytes)
+      return fail(VR_ERR_UNALIGNED, "rank " + std::to_string(r));
+    int rc = calc_work_size(0, nelems * 2, 1, (size_t)a->msg_bytes, &work);
+    if (rc) return fail(rc, "nelems " + std::to_string(nelems));
+  }
+  if (work_bytes) *work_bytes = work;
+  return VR_OK;
+}
+
+extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geometry *out) {
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || !out) return fail(VR_ERR_INVALID, "bad algo or null output");
+  if (int rc = check_topology(a, nranks)) return rc;
+  // getLaunchParam (allreduce.hpp:37-62, 237-258; allgather.hpp:32-56), PVC constants.
+  const size_t n_threads = 64, max_ss = 64;
+  const size_t w = (a->transmit == T_PARALLEL || a->transmit == T_BISECT) ? (size_t)nranks : 1;
+  const size_t work = a->allgather ? nelems * 2 : nelems * 2 / (size_t)nranks;
+  const size_t wire_per_ss = n_threads / w;
+  const size_t n_wire = div_up(work, (size_t)a->wire_capacity);
+  const size_t n_ss = div_up(n_wire, wire_per_ss);
+  const size_t actual_ss = n_ss < max_ss ? n_ss : max_ss;
+  out->steps = actual_ss ? (uint32_t)div_up(n_wire, actual_ss * wire_per_ss) : 0;
+  out->subgroups = (uint32_t)(wire_per_ss * w);
+  out->groups = (uint32_t)actual_ss;
+  return VR_OK;
+}
+
+// ---------------------------------------------------------------------------------
+// context
+// ---------------------------------------------------------------------------------
+
+struct vr_ctx {
+  int nranks = 0;
+  DeviceInfo dev;
+  Tuning tuning;
+  bool tuning_user_block = false;
+  uint32_t seq_no = 1;
+  uint64_t spin_limit = 0;
+};
+
+extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
+  if (!out) return fail(VR_ERR_INVALID, "null out");
+  *out = nullptr;
+  if (!(nranks == 2 || nranks == 4 || nranks == 8 || nranks == 16))
+    return fail(VR_ERR_TOPOLOGY, "nranks must be 2, 4, 8 or 16");
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count == 0) {
+    (void)hipGetLastError();
+    return fail(VR_ERR_NO_DEVICE, "no HIP device visible");
+  }
+  if (device < 0 || device >= count) return fail(VR_ERR_INVALID, "device index out of range");
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(VR_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", kernels are built for gfx950");
+  vr_ctx *c = new vr_ctx;
+  c->nranks = nranks;
+  c->dev.device = device;
+  c->dev.cus = prop.multiProcessorCount;
+  snprintf(c->dev.arch, sizeof c->dev.arch, "%s", prop.gcnArchName);
+  HIP_TRY(hipSetDevice(device));
+  *out = c;
+  return VR_OK;
+}
+
+extern "C" int vr_ctx_destroy(vr_ctx *ctx) {
+  if (!ctx) return VR_OK;
+  delete ctx;
+  return VR_OK;
+}
+
+extern "C" int vr_ctx_nranks(const vr_ctx *ctx) { return ctx ? ctx->nranks : 0; }
+
+extern "C" int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  ctx->spin_limit = polls;
+  return VR_OK;
+}
+
+static int *tuning_field(vr_ctx *ctx, const char *key) {
+  if (!ctx || !key) return nullptr;
+  if (!strcmp(key, "block")) return &ctx->tuning.block;
+  if (!strcmp(key, "waves_per_cu")) return &ctx->tuning.waves_per_cu;
+  if (!strcmp(key, "unroll")) return &ctx->tuning.unroll;
+  if (!strcmp(key, "nt_load")) return &ctx->tuning.nt_load;
+  if (!strcmp(key, "nt_store")) return &ctx->tuning.nt_store;
+  if (!strcmp(key, "oneshot")) return &ctx->tuning.oneshot;
+  return nullptr;
+}
+
+extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
+  int *f = tuning_field(ctx, key);
+  if (!f) return fail(VR_ERR_INVALID, std::string("unknown tuning key ") + (key ? key : "(null)"));
+  if (!strcmp(key, "block") && (value < 64 || value > 1024 || value % 64))
+    return fail(VR_ERR_INVALID, "block must be a multiple of 64 in [64,1024]");
+  if (!strcmp(key, "waves_per_cu") && (value < 1 || value > 64))
+    return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
+  if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
+    return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
+  *f = value;
+  return VR_OK;
+}
+
+extern "C" int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value) {
+  int *f = tuning_field(ctx, key);
+  if (!f || !value) return fail(VR_ERR_INVALID, "unknown tuning key");
+  *value = *f;
+  return VR_OK;
+}
+
+// ---------------------------------------------------------------------------------
+// hot path
+// ---------------------------------------------------------------------------------
+
+static bool ranges_partially_overlap(const void *a, const void *b, size_t bytes) {
+  if (a == b) return false;
+  const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
+  return x < y + bytes && y < x + bytes;
+}
+
+static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a) {
+  Tuning t = ctx->tuning;
+  if (a->latency_tuned) {
+    // "small" family: every lane makes one trip, results stay cacheable for
+    // the kernel that consumes them next.
+    t.oneshot = 1;
+    t.unroll = 1;
+    t.nt_load = 0;
+    t.nt_store = 0;
+    t.block = 256;
+  }
+  return t;
+}
+
+struct Prepared {
+  const AlgoInfo *a;
+  PtrTable in, out;
+  size_t chunk_elems;
+  int vec_halves;
+  vr_geometry geom;
+};
+
+static int prepare_allreduce(vr_ctx *ctx, int algo, void *const bufs[], void *const outs[],
+                             size_t nelems, Prepared *p) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
+  const int N = ctx->nranks;
+  size_t work = 0;
+  if (int rc = vr_check_allreduce(algo, N, (const void *const *)bufs, nelems, &work)) return rc;
+  if (outs) {
+    if (int rc = vr_check_allreduce(algo, N, (const void *const *)outs, nelems, &work)) return rc;
+    for (int r = 0; r < N; ++r)
+      for (int q = 0; q < N; ++q) {
+        if (ranges_partially_overlap(outs[r], bufs[q], nelems * 2))
+          return fail(VR_ERR_OVERLAP, "outs[" + std::to_string(r) + "] vs bufs[" + std::to_string(q) + "]");
+        if (r != q && ranges_partially_overlap(outs[r], outs[q], nelems * 2))
+          return fail(VR_ERR_OVERLAP, "outs[" + std::to_string(r) + "] vs outs[" + std::to_string(q) + "]");
+      }
+  }
+  p->a = a;
+  memset(&p->in, 0, sizeof p->in);
+  memset(&p->out, 0, sizeof p->out);
+  bool align16 = true;
+  for (int r = 0; r < N; ++r) {
+    p->in.p[r] = bufs[r];
+    p->out.p[r] = outs ? outs[r] : bufs[r];
+    align16 = align16 && ((uintptr_t)p->in.p[r] % 16 == 0) && ((uintptr_t)p->out.p[r] % 16 == 0);
+  }
+  p->chunk_elems = work / 2;
+  p->vec_halves = (align16 && p->chunk_elems % 8 == 0) ? 8 : 4;
+  return vr_launch_geometry(algo, N, nelems, &p->geom);
+}
+
+static int resolve_transport(const AlgoInfo *a, int transport, int *out) {
+  if (transport == VR_TRANSPORT_DEFAULT)
+    transport = (a == &kAlgos[VR_ALGO_PARALLEL]) ? VR_TRANSPORT_WIRE : VR_TRANSPORT_DIRECT;
+  if (transport != VR_TRANSPORT_DIRECT && transport != VR_TRANSPORT_WIRE)
+    return fail(VR_ERR_INVALID, "bad transport");
+  *out = transport;
+  return VR_OK;
+}
+
+static int run_allreduce(vr_ctx *ctx, hipStream_t s, const Prepared &p, int transport,
+                         const Tuning &t, uint32_t seq_no) {
+  (void)seq_no;
+  if (transport == VR_TRANSPORT_WIRE)
+    return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
+  hipError_t e = launch_direct_allreduce(s, ctx->dev, t, ctx->nranks, p.a->order, p.in, p.out,
+                                         p.chunk_elems, p.vec_halves);
+  if (e != hipSuccess) return fail_hip(e, "launch_direct_allreduce");
+  return VR_OK;
+}
+
+extern "C" int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                            void *const outs[], size_t nelems, uint32_t *seq_no) {
+  Prepared p;
+  if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
+  int tr;
+  if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
+  uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
+  const uint32_t start = *seq;
+  if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr, tuning_for(ctx, p.a), start)) return rc;
+  *seq = start + p.geom.steps;   // getLaunchParam: updateSeqNo += nSteps
+  return VR_OK;
+}
+
+extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transport,
+                                 void *const bufs[], void *const outs[], size_t nelems,
+                                 uint32_t seq_no, uint32_t groups, uint32_t subgroups,
+                                 uint32_t simd) {
+  // main.cpp:289-291, then allreduce.cpp:852/917.
+  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
+  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
+  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
+  Prepared p;
+  if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
+  int tr;
+  if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
+  // Map the reference's (groups x subgroups x simd) grid onto wavefronts: a block
+  // holds the same number of lanes (rounded to whole waves, at most 1024) and the
+  // launch holds ceil(groups / nranks) blocks for every virtual rank.
+  Tuning t = ctx->tuning;
+  size_t lanes = (size_t)subgroups * simd;
+  lanes = ((lanes + 63) / 64) * 64;
+  if (lanes > 1024) lanes = 1024;
+  t.block = (int)lanes;
+  t.unroll = 1;
+  t.oneshot = 0;
+  t.force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
+  return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no);
+}
+
+struct PreparedGather {
+  const AlgoInfo *a;
+  PtrTable in, out;
+  int vec_halves;
+  vr_geometry geom;
+};
+
+static int prepare_allgather(vr_ctx *ctx, int algo, const void *const inputs[],
+                             void *const outputs[], size_t nelems, PreparedGather *p) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
+  const int N = ctx->nranks;
+  if (int rc = vr_check_allgather(algo, N, inputs, outputs, nelems, nullptr)) return rc;
+  const size_t bytes = nelems * 2;
+  for (int r = 0; r < N; ++r)
+    for (int q = 0; q < N; ++q) {
+      // input q may be exactly slot q of output r == q; anything else must be disjoint
+      const char *slot_q = (const char *)outputs[r] + (size_t)q * bytes;
+      const bool same = (const void *)slot_q == inputs[q];
+      const uintptr_t x = (uintptr_t)inputs[q], y = (uintptr_t)outputs[r];
+      const bool overlap = x < y + bytes * N && y < x + bytes;
+      if (overlap && !same) return fail(VR_ERR_OVERLAP, "outputs[" + std::to_string(r) + "] vs inputs[" + std::to_string(q) + "]");
+      if (r != q) {
+        const uintptr_t z = (uintptr_t)outputs[q];
+        if (z < y + bytes * N && y < z + bytes * N) return fail(VR_ERR_OVERLAP, "outputs overlap");
+      }
+    }
+  p->a = a;
+  memset(&p->in, 0, sizeof p->in);
+  memset(&p->out, 0, sizeof p->out);
+  bool align16 = true;
+  for (int r = 0; r < N; ++r) {
+    p->in.p[r] = const_cast<void *>(inputs[r]);
+    p->out.p[r] = outputs[r];
+    align16 = align16 && ((uintptr_t)inputs[r] % 16 == 0) && ((uintptr_t)outputs[r] % 16 == 0);
+  }
+  p->vec_halves = (align16 && nelems % 8 == 0) ? 8 : 4;
+  // An 8-byte-granular tail cannot occur: the all-gather messages are 16 bytes.
+  return vr_launch_geometry(algo, N, nelems, &p->geom);
+}
+
+extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
+                            const void *const inputs[], void *const outputs[], size_t nelems,
+                            uint32_t *seq_no) {
+  PreparedGather p;
+  if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
+  if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
+  if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
+  hipError_t e = launch_direct_allgather((hipStream_t)stream, ctx->dev, tuning_for(ctx, p.a),
+                                         ctx->nranks, p.in, p.out, nelems, p.vec_halves);
+  if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
+  uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
+  *seq += p.geom.steps;
+  return VR_OK;
+}
+
+extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return VR_OK;
+}
+
+// ---------------------------------------------------------------------------------
+// timing
+// ---------------------------------------------------------------------------------
+
+template <typename F>
+static int time_launches(hipStream_t s, int iters, float *ms_out, F &&launch) {
+  if (iters <= 0 || !ms_out) return fail(VR_ERR_INVALID, "iters <= 0 or null ms_out");
+  const int kBatch = 128;   // events in flight before the host waits
+  std::vector<hipEvent_t> ev(2 * (size_t)kBatch);
+  for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+  int rc = VR_OK;
+  for (int done = 0; done < iters && rc == VR_OK; done += kBatch) {
+    const int n = (iters - done < kBatch) ? iters - done : kBatch;
+    for (int i = 0; i < n && rc == VR_OK; ++i) {
+      if (hipEventRecord(ev[2 * i], s) != hipSuccess) rc = fail(VR_ERR_HIP, "hipEventRecord");
+      if (rc == VR_OK) rc = launch();
+      if (rc == VR_OK && hipEventRecord(ev[2 * i + 1], s) != hipSuccess) rc = fail(VR_ERR_HIP, "hipEventRecord");
+    }
+    if (rc != VR_OK) break;
+    hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) { rc = fail_hip(e, "hipStreamSynchronize"); break; }
+    for (int i = 0; i < n; ++i) {
+      float ms = 0.f;
+      e = hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]);
+      if (e != hipSuccess) { rc = fail_hip(e, "hipEventElapsedTime"); break; }
+      ms_out[done + i] = ms;
+    }
+  }
+  for (auto &e : ev) (void)hipEventDestroy(e);
+  return rc;
+}
+
+extern "C" int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transport,
+                                 void *const bufs[], void *const outs[], size_t nelems, int iters,
+                                 float *ms_out) {
+  Prepared p;
+  if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
+  int tr;
+  if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
+  const Tuning t = tuning_for(ctx, p.a);
+  hipStream_t s = (hipStream_t)stream;
+  return time_launches(s, iters, ms_out, [&]() -> int {
+    const uint32_t start = ctx->seq_no;
+    int rc = run_allreduce(ctx, s, p, tr, t, start);
+    ctx->seq_no = start + p.geom.steps;
+    return rc;
+  });
+}
+
+extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
+                                 const void *const inputs[], void *const outputs[], size_t nelems,
+                                 int iters, float *ms_out) {
+  PreparedGather p;
+  if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
+  if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
+  const Tuning t = tuning_for(ctx, p.a);
+  hipStream_t s = (hipStream_t)stream;
+  return time_launches(s, iters, ms_out, [&]() -> int {
+    hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);
+    return e == hipSuccess ? VR_OK : fail_hip(e, "launch_direct_allgather");
+  });
+}
+
+extern "C" int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes,
+                            int iters, float *ms_out) {
+  if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
+  if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16) return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
+  hipStream_t s = (hipStream_t)stream;
+  return time_launches(s, iters, ms_out, [&]() -> int {
+    hipError_t e = launch_copy(s, ctx->dev, ctx->tuning, dst, src, bytes);
+    return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
+  });
+}
+
+// ---------------------------------------------------------------------------------
+// host helpers
+// ---------------------------------------------------------------------------------
+
+// double -> binary16, one rounding (round-to-nearest-even), overflow to infinity.
+static uint16_t f64_to_f16(double d) {
+  if (d != d) return 0x7e00;
+  const uint16_t sign = signbit(d) ? 0x8000 : 0;
+  const double a = fabs(d);
+  if (a >= 65520.0) return (uint16_t)(sign | 0x7c00);
+  if (a == 0.0) return sign;
+  int ex;
+  (void)frexp(a, &ex);
+  int e = ex - 1;
+  if (e < -14) e = -14;
+  const uint32_t q = (uint32_t)nearbyint(ldexp(a, 10 - e));
+  uint32_t bits = (e == -14 && q < 1024) ? q : (((uint32_t)(e + 15) << 10) + q - 1024);
+  if (bits >= 0x7c00) bits = 0x7c00;
+  return (uint16_t)(sign | bits);
+}
+
+extern "C" void vr_fill_pattern(uint16_t *host_buf, int rank, size_t n) {
+  for (size_t i = 0; i < n; ++i) host_buf[i] = f64_to_f16((double)((int)(i % 32) * (rank + 1)));
+}
+
+static inline uint64_t splitmix64_at(uint64_t seed, uint64_t k) {
+  uint64_t z = seed + (k + 1) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+extern "C" void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dist, double p0,
+                            double p1) {
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t z0 = splitmix64_at(seed, 2 * (uint64_t)i);
+    const uint64_t z1 = splitmix64_at(seed, 2 * (uint64_t)i + 1);
+    double x;
+    if (dist == 0) {
+      x = p0 + (p1 - p0) * ((double)(z0 >> 11) * 0x1.0p-53);
+    } else {
+      const double u1 = (double)((z0 >> 11) + 1) * 0x1.0p-53;
+      const double u2 = (double)(z1 >> 11) * 0x1.0p-53;
+      x = p0 + p1 * (sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2));
+    }
+    host_buf[i] = f64_to_f16(x);
+  }
+}
+
+extern "C" int vr_parse_nelems(const char *text, size_t *out) {
+  if (!text || !out) return fail(VR_ERR_INVALID, "null argument");
+  // main.cpp:17-34: the last K / M / G anywhere in the string picks the base,
+  // the leading digits are the count ("8MB" -> 8 * 1024 * 1024).
+  size_t base = 1;
+  if (strrchr(text, 'K')) base = 1024ull;
+  else if (strrchr(text, 'M')) base = 1024ull * 1024;
+  else if (strrchr(text, 'G')) base = 1024ull * 1024 * 1024;
+  char *end = nullptr;
+  const unsigned long long v = strtoull(text, &end, 10);
+  if (end == text) return fail(VR_ERR_INVALID, std::string("no digits in '") + text + "'");
+  *out = (size_t)v * base;
+  return VR_OK;
+}
+
+extern "C" int vr_device_count(int *count) {
+  if (!count) return fail(VR_ERR_INVALID, "null argument");
+  if (hipGetDeviceCount(count) != hipSuccess) {
+    (void)hipGetLastError();
+    *count = 0;
+  }
+  return VR_OK;
+}
+
+extern "C" int vr_device_name(int device, char *buf, size_t buflen) {
+  if (!buf || !buflen) return fail(VR_ERR_INVALID, "null argument");
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  snprintf(buf, buflen, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  return VR_OK;
+}
+
+extern "C" int vr_malloc(int device, size_t bytes, void **out) {
+  if (!out) return fail(VR_ERR_INVALID, "null argument");
+  HIP_TRY(hipSetDevice(device));
+  HIP_TRY(hipMalloc(out, bytes ? bytes : 16));
+  return VR_OK;
+}
+
+extern "C" int vr_free(void *ptr) {
+  if (ptr) HIP_TRY(hipFree(ptr));
+  return VR_OK;
+}
+
+extern "C" int vr_memset(void *ptr, int value, size_t bytes) {
+  HIP_TRY(hipMemset(ptr, value, bytes));
+  return VR_OK;
+}
+
+extern "C" int vr_copy_to_device(void *dst, const void *src_host, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst, src_host, bytes, hipMemcpyHostToDevice));
+  return VR_OK;
+}
+
+extern "C" int vr_copy_to_host(void *dst_host, const void *src, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst_host, src, bytes, hipMemcpyDeviceToHost));
+  return VR_OK;
+}
+
+extern "C" int vr_stream_create(int device, void **stream_out) {
+  if (!stream_out) return fail(VR_ERR_INVALID, "null argument");
+  HIP_TRY(hipSetDevice(device));
+  hipStream_t s;
+  HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream_out = s;
+  return VR_OK;
+}
+
+extern "C" int vr_stream_destroy(void *stream) {
+  if (stream) HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+  return VR_OK;
+}
+
+extern "C" int vr_stream_sync(void *stream) {
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return VR_OK;
+}

@@ -1,0 +1,209 @@
+/*
+ * vrank_allreduce.h — C ABI of the MI355X single-shot all-reduce / all-gather
+ * data path over "virtual ranks" (NRanks separate device allocations in one
+ * GPU's HBM).
+ *
+ * This is the boundary a host program binds instead of the reference's SYCL
+ * functors.  Plain pointers and sizes only; every function returns a vr_status
+ * (0 = success) and never throws.  The C++ header vrank/allreduce.hpp turns the
+ * codes back into the reference's std::logic_error texts.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   vr_allreduce      <- AllReduce<T,N,Proto,Transmit>::launch       allreduce.hpp:64-74
+ *                        bisectPAllReduce<T,N>::launch               allreduce.hpp:260-270
+ *                        testTransmit<T>(std::string algo, ...)      allreduce.cpp:1118-1189
+ *   vr_allgather      <- AllGather<T,N,Proto,Transmit>::launch       allgather.hpp:58-70
+ *                        testAllgather<T>(std::string algo, ...)     allreduce.cpp:1191-1213
+ *   vr_check_allreduce<- AllReduce::calcWorkSize                     allreduce.hpp:108-122
+ *   vr_check_allgather<- AllGather::calcWorkSize                     allgather.hpp:104-117
+ *   vr_launch_geometry<- AllReduce::getLaunchParam                   allreduce.hpp:37-62, 237-258
+ *   vr_algo_from_string<- the -a string switch                       allreduce.cpp:1128-1188, 1198-1212
+ *   vr_fill_pattern   <- fill_pattern                                utils.hpp:15-19
+ *   vr_parse_nelems   <- parse_nelems                                main.cpp:17-34
+ *   vr_ctx_create     <- scratch allocation + zeroing + peer tables  main.cpp:224-283
+ *                        (Level Zero IPC exchange, ipc_exchange.cpp, has no
+ *                        counterpart: all virtual ranks live in one address space)
+ */
+#ifndef VRANK_ALLREDUCE_H
+#define VRANK_ALLREDUCE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VR_MAX_RANKS 16
+
+typedef enum vr_status {
+  VR_OK = 0,
+  VR_ERR_UNALIGNED = 1,   /* "We only support aligned pointer for now"      allreduce.hpp:111 */
+  VR_ERR_UNEVEN = 2,      /* "We don't support non-even divide yet"         allreduce.hpp:118 */
+  VR_ERR_ALGO = 3,        /* "Transmit type not support"                    allreduce.cpp:1187 */
+  VR_ERR_TOPOLOGY = 4,    /* "Unsupported communication topology"           allreduce.cpp:880  */
+  VR_ERR_SUBGROUP = 5,    /* "Unsupported Sub-group size"                   allreduce.cpp:917  */
+  VR_ERR_GEOMETRY = 6,    /* "Subgroup numbers must be multiple of 4"       main.cpp:289-291   */
+  VR_ERR_INVALID = 7,     /* null pointer / bad enum / size beyond what the context was built for */
+  VR_ERR_HIP = 8,         /* a HIP runtime call failed; see vr_last_error_detail()             */
+  VR_ERR_NO_DEVICE = 9,   /* no gfx950 device visible                                          */
+  VR_ERR_TIMEOUT = 10,    /* a flag poll in the wire transport exceeded its spin limit         */
+  VR_ERR_OVERLAP = 11,    /* out-of-place buffers alias in a way the kernel cannot honour      */
+} vr_status;
+
+/* The -a strings of the reference (README.md:18, allreduce.cpp:1128-1212) plus
+ * "parallel" (ParallelTransmit named directly). */
+typedef enum vr_algo {
+  VR_ALGO_SMALL = 0,            /* Rt64          + ParallelTransmit   */
+  VR_ALGO_SIMPLE = 1,           /* Rt64_128      + ParallelTransmit   */
+  VR_ALGO_BISECT = 2,           /* BisectPTransmit                    */
+  VR_ALGO_PARALLEL = 3,         /* ParallelTransmit, message-passing form (see vr_transport) */
+  VR_ALGO_SMALL_PCIE_P = 4,     /* Rt64_PCIE     + ParallelTransmit   */
+  VR_ALGO_SIMPLE_PCIE_P = 5,    /* Rt64_128_PCIE + ParallelTransmit   */
+  VR_ALGO_SMALL_RING = 6,       /* Rt64_PCIE     + RingTransmit       */
+  VR_ALGO_SIMPLE_RING = 7,      /* Rt64_128_PCIE + RingTransmit       */
+  VR_ALGO_SMALL_PCIE = 8,       /* Rt64_PCIE     + SequentialTransmit */
+  VR_ALGO_SIMPLE_PCIE = 9,      /* Rt64_128_PCIE + SequentialTransmit */
+  VR_ALGO_ALLGATHER_SMALL = 10, /* Rt64_PCIE     + RingTransmit::runAllgather */
+  VR_ALGO_ALLGATHER_SIMPLE = 11,/* Rt64_128_PCIE + RingTransmit::runAllgather */
+  VR_ALGO_COUNT_
+} vr_algo;
+
+/* How data travels between virtual ranks.
+ *  DIRECT: the workgroups of the rank that owns a chunk read every rank's input
+ *          in place, add in the protocol's order, and write every rank's output.
+ *          One pass over HBM; no scratch, no flags.  Default for every algo
+ *          except VR_ALGO_PARALLEL.
+ *  WIRE  : the reference's stage structure — scatter into the owner's sink,
+ *          reduce, gather into every peer's sink — through the context's scratch
+ *          with agent-scope release/acquire flag words, one persistent kernel
+ *          whose workgroups are partitioned between the virtual ranks.  This is
+ *          the form that carries over to several GPUs.  Default for
+ *          VR_ALGO_PARALLEL. */
+typedef enum vr_transport {
+  VR_TRANSPORT_DEFAULT = 0,
+  VR_TRANSPORT_DIRECT = 1,
+  VR_TRANSPORT_WIRE = 2,
+} vr_transport;
+
+typedef struct vr_ctx vr_ctx;
+
+/* ---- lifetime --------------------------------------------------------------- */
+
+/* Creates a context for `nranks` virtual ranks on HIP device `device`.  Allocates
+ * (and zeroes once, main.cpp:251) the wire-transport scratch: per rank a scatter
+ * and a gather region plus flag words.  nranks must be 2, 4, 8 or 16. */
+int vr_ctx_create(int device, int nranks, vr_ctx **out);
+int vr_ctx_destroy(vr_ctx *ctx);
+int vr_ctx_nranks(const vr_ctx *ctx);
+
+/* ---- validation (host only, no GPU needed) ------------------------------------ */
+
+int vr_algo_from_string(const char *name, int *algo_out);        /* VR_ERR_ALGO if unknown */
+const char *vr_algo_name(int algo);
+int vr_algo_is_allgather(int algo);
+size_t vr_algo_message_bytes(int algo);                          /* sizeof(message_t): 8 or 16 */
+
+/* calcWorkSize: pointer alignment and even divisibility for an all-reduce of
+ * `nelems` halves per rank.  *work_bytes (optional) = bytes per rank-chunk. */
+int vr_check_allreduce(int algo, int nranks, const void *const bufs[], size_t nelems,
+                       size_t *work_bytes);
+int vr_check_allgather(int algo, int nranks, const void *const inputs[], void *const outputs[],
+                       size_t nelems, size_t *work_bytes);
+
+/* getLaunchParam: the grid the reference would pick for this size, and how far
+ * it advances the sequence number. */
+typedef struct vr_geometry {
+  uint32_t groups;        /* work-groups                              */
+  uint32_t subgroups;     /* sub-groups (16 lanes) per work-group     */
+  uint32_t steps;         /* loop steps each wire makes = seqNo bump  */
+} vr_geometry;
+int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geometry *out);
+
+/* ---- the hot path ------------------------------------------------------------ */
+
+/* All-reduce of `nelems` binary16 values per rank across ctx's virtual ranks.
+ *   bufs[r]  : rank r's input (device memory, message-aligned).
+ *   outs     : NULL for the reference's in-place semantics (bufs[r] receives the
+ *              sum), or N output pointers (outs[r] may equal bufs[r]).
+ *   seq_no   : in/out sequence number, advanced like getLaunchParam does; only the
+ *              wire transport consumes it.  May be NULL (context keeps its own).
+ * Asynchronous on `stream` (a hipStream_t; NULL = the null stream).  The sum is
+ * bit-identical to the reference kernels' order for `algo`: rotated chain from
+ * the chunk owner (all but bisect), pair tree (bisect). */
+int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                 void *const outs[], size_t nelems, uint32_t *seq_no);
+
+/* All-gather: outputs[r][p*nelems + i] = inputs[p][i] for every rank r.
+ * outputs[r] + r*nelems may alias inputs[r] (sequential_transmit.hpp:496-497). */
+int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void *const inputs[],
+                 void *const outputs[], size_t nelems, uint32_t *seq_no);
+
+/* Reference test-harness flavour (testTransmit with a user grid, main.cpp:289-314):
+ * `groups` x `subgroups` sub-groups of `simd` lanes.  Results never depend on the
+ * grid; unusable grids are rejected the way the reference's host code rejects
+ * them (VR_ERR_GEOMETRY / VR_ERR_SUBGROUP). */
+int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                      void *const outs[], size_t nelems, uint32_t seq_no, uint32_t groups,
+                      uint32_t subgroups, uint32_t simd);
+
+/* After a wire-transport launch has completed: VR_OK, or VR_ERR_TIMEOUT if any
+ * poll gave up.  (Synchronises `stream`.) */
+int vr_ctx_check(vr_ctx *ctx, void *stream);
+/* Poll budget of the wire transport's bounded spin (0 = library default). */
+int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
+
+/* Tuning knobs for the direct kernels (benchmark sweeps).  Unknown keys are
+ * VR_ERR_INVALID.  Keys: "block" (threads per work-group), "waves_per_cu"
+ * (persistent grid size = CUs * this / waves per block), "unroll" (16-byte
+ * vectors in flight per lane and rank), "nt_load", "nt_store" (0/1). */
+int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value);
+int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);
+
+/* ---- timing ------------------------------------------------------------------- */
+
+/* Launches the all-reduce `iters` times on `stream`, each bracketed by its own
+ * pair of HIP events recorded on that stream, and returns the per-launch kernel
+ * times in milliseconds (ms_out[iters]).  Out-of-place when outs != NULL. */
+int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                      void *const outs[], size_t nelems, int iters, float *ms_out);
+int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
+                      const void *const inputs[], void *const outputs[], size_t nelems, int iters,
+                      float *ms_out);
+/* Plain device copy of `bytes` (dwordx4 loads, nontemporal stores) timed the
+ * same way: the practical HBM ceiling next to which the all-reduce is read. */
+int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int iters,
+                 float *ms_out);
+
+/* ---- host helpers -------------------------------------------------------------- */
+
+void vr_fill_pattern(uint16_t *host_buf, int rank, size_t n);     /* utils.hpp:15-19 */
+/* Seeded data: dist 0 = uniform [p0,p1), 1 = normal(mean p0, sd p1); splitmix64
+ * keyed by seed, element i from draws 2i, 2i+1; rounded once to binary16. */
+void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dist, double p0, double p1);
+/* "8MB" -> 8*1024*1024, "64K", "2G", plain digits (main.cpp:17-34). */
+int vr_parse_nelems(const char *text, size_t *out);
+
+/* Thin device-memory plumbing so that C, Python (ctypes) and the CLI need no
+ * other GPU runtime binding. */
+int vr_device_count(int *count);
+int vr_device_name(int device, char *buf, size_t buflen);
+int vr_malloc(int device, size_t bytes, void **out);
+int vr_free(void *ptr);
+int vr_memset(void *ptr, int value, size_t bytes);
+int vr_copy_to_device(void *dst, const void *src_host, size_t bytes);
+int vr_copy_to_host(void *dst_host, const void *src, size_t bytes);
+int vr_stream_create(int device, void **stream_out);
+int vr_stream_destroy(void *stream);
+int vr_stream_sync(void *stream);
+
+/* ---- errors ---------------------------------------------------------------------- */
+
+const char *vr_strerror(int status);          /* the reference's exception text where one exists */
+const char *vr_last_error_detail(void);       /* thread-local detail of the last non-zero status */
+const char *vr_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VRANK_ALLREDUCE_H */

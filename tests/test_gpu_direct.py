@@ -1,0 +1,293 @@
+"""GPU parity tests (direct transport): HIP path through the C ABI vs the CPU
+oracle on the same seeded inputs.  Bit-exact: binary16 sums must match in every
+bit (NaNs compare equal to NaNs)."""
+import numpy as np
+import pytest
+
+import gpu_ipc_example_amd as vr
+from tests import vr_helpers as H
+from tests.oracle_lib import DIST_NORMAL, DIST_UNIFORM
+
+pytestmark = pytest.mark.gpu
+
+
+def h(x):
+    return int(np.array([x], np.float16).view(np.uint16)[0])
+
+
+@pytest.fixture(scope="module")
+def ctxs():
+    made = {n: vr.VirtualRanks(n) for n in (2, 4, 8, 16)}
+    yield made
+    for c in made.values():
+        c.close()
+
+
+def per_chunk(out, nranks):
+    chunk = len(out) // nranks
+    vals = []
+    for c in range(nranks):
+        seg = out[c * chunk:(c + 1) * chunk].view(np.float16)
+        assert (seg == seg[0]).all()
+        vals.append(float(seg[0]))
+    return vals
+
+
+# ---- known answers that separate the summation orders -------------------------------
+
+def test_kat_n4(ctxs):
+    ins = [np.full(256, h(v), np.uint16) for v in (2048, 1, 1, 0)]
+    got, _ = H.run_allreduce(ctxs[4], "simple", ins)
+    for g in got:
+        assert per_chunk(g, 4) == [2048, 2050, 2048, 2048]
+    got, _ = H.run_allreduce(ctxs[4], "bisect", ins)
+    for g in got:
+        assert per_chunk(g, 4) == [2048, 2048, 2048, 2048]
+    ins = [np.full(256, h(v), np.uint16) for v in (1, 1, 2048, 0)]
+    got, _ = H.run_allreduce(ctxs[4], "bisect", ins)
+    for g in got:
+        assert per_chunk(g, 4) == [2050, 2050, 2050, 2050]
+
+
+@pytest.mark.parametrize("algo", ["small", "simple", "bisect", "small_ring", "simple_pcie"])
+def test_kat_n8_three_way(ctxs, algo):
+    ins = [np.full(1024, h(v), np.uint16) for v in (2048, 0, 1, 0, 1, 0, 0, 0)]
+    got, _ = H.run_allreduce(ctxs[8], algo, ins)
+    want = ([2048, 2050, 2048, 2048, 2048, 2050, 2048, 2048] if algo == "bisect"
+            else [2048, 2050, 2050, 2048, 2048, 2048, 2048, 2048])
+    for g in got:
+        assert per_chunk(g, 8) == want
+
+
+# ---- the reference's own fixture and shape list ----------------------------------------
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+def test_fill_pattern_shapes(ctxs, oracle, nranks):
+    for n in (128, 256, 384, 1280, 1920, 1024, 2048, 14336, 16384):   # test_2tile_shapes.sh:4
+        ins = [oracle.fill_pattern(r, n) for r in range(nranks)]
+        want = ((np.arange(n) % 32) * (nranks * (nranks + 1) // 2)).astype(np.float16).view(np.uint16)
+        for algo in ("small", "simple") + (("bisect",) if nranks >= 4 else ()):
+            if n % (4 * nranks):
+                continue
+            got, _ = H.run_allreduce(ctxs[nranks], algo, ins)
+            H.assert_all_ranks_equal(oracle, got, want, "%s n=%d" % (algo, n))
+
+
+@pytest.mark.parametrize("groups", [1, 2, 4, 8, 16, 32, 64, 7, 13, 15, 17, 19])
+def test_result_independent_of_grid(ctxs, oracle, groups):
+    """test_8tile_shapes.sh sweeps -g x -w; sub-group counts are kept to the
+    multiples of 4 that main.cpp:289-291 still accepts."""
+    n = 14336
+    ins = H.make_inputs(oracle, 8, n, 500)
+    for algo in ("small", "bisect"):
+        want = H.expected(oracle, algo, ins)
+        for subgroups in (4, 8, 32, 64):
+            got, _ = H.run_allreduce(ctxs[8], algo, ins, grid=(groups, subgroups, 16))
+            H.assert_all_ranks_equal(oracle, got, want, "%s g=%d w=%d" % (algo, groups, subgroups))
+
+
+def test_grid_validation(ctxs, oracle):
+    ins = H.make_inputs(oracle, 8, 1024, 1)
+    for bad_w in (1, 2, 6):
+        with pytest.raises(vr.VRError) as e:
+            H.run_allreduce(ctxs[8], "small", ins, grid=(4, bad_w, 16))
+        assert e.value.code == "GEOMETRY"
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[8], "small", ins, grid=(4, 4, 8))
+    assert e.value.code == "SUBGROUP"
+    got, _ = H.run_allreduce(ctxs[8], "small", ins, grid=(4, 4, 32))
+    H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins))
+
+
+# ---- random data, every algo string, every world size --------------------------------------
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("algo", H.ROTATED_ALGOS + ("bisect",))
+def test_random_all_algos(ctxs, oracle, nranks, algo):
+    if algo == "bisect" and nranks < 4:
+        pytest.skip("bisect needs >= 4 ranks")
+    msg = 16 if ("pcie" in algo or "ring" in algo) else 8
+    unit = (msg // 2) * nranks
+    for k, n in enumerate((unit, unit * 3, unit * 129, unit * 1000 + unit, 1 << 20)):
+        if n % unit:
+            n = (n // unit) * unit
+        ins = H.make_inputs(oracle, nranks, n, 1000 * nranks + 10 * k)
+        want = H.expected(oracle, algo, ins)
+        got, _ = H.run_allreduce(ctxs[nranks], algo, ins)
+        H.assert_all_ranks_equal(oracle, got, want, "%s N=%d n=%d in-place" % (algo, nranks, n))
+        got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=False)
+        H.assert_all_ranks_equal(oracle, got, want, "%s N=%d n=%d out-of-place" % (algo, nranks, n))
+        for a, b in zip(kept, ins):
+            assert (a == b).all(), "out-of-place run modified an input"
+
+
+def test_bisect_16_ranks(ctxs, oracle):
+    for n in (64, 64 * 77, 1 << 18):
+        ins = H.make_inputs(oracle, 16, n, 77)
+        got, _ = H.run_allreduce(ctxs[16], "bisect", ins)
+        H.assert_all_ranks_equal(oracle, got, oracle.bisect(ins))
+
+
+@pytest.mark.parametrize("algo", ["simple", "bisect"])
+def test_eight_byte_granularity(ctxs, oracle, algo):
+    """Chunks that are a multiple of 8 bytes but not of 16, and pointers that are
+    only 8-byte aligned: both legal for the 8-byte message protocols."""
+    for n in (32 * 1, 32 * 3, 32 * 1001):                 # chunk = 4, 12, 4004 halves
+        ins = H.make_inputs(oracle, 8, n, 40 + n)
+        want = H.expected(oracle, algo, ins)
+        got, _ = H.run_allreduce(ctxs[8], algo, ins)
+        H.assert_all_ranks_equal(oracle, got, want, "n=%d" % n)
+    ins = H.make_inputs(oracle, 8, 1 << 16, 9)
+    want = H.expected(oracle, algo, ins)
+    got, _ = H.run_allreduce(ctxs[8], algo, ins, offset_bytes=8)
+    H.assert_all_ranks_equal(oracle, got, want, "offset 8")
+    got, _ = H.run_allreduce(ctxs[8], algo, ins, offset_bytes=8, inplace=False)
+    H.assert_all_ranks_equal(oracle, got, want, "offset 8 out-of-place")
+
+
+def test_runtime_rejections(ctxs, oracle):
+    ins = H.make_inputs(oracle, 8, 1 << 12, 3)
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[8], "simple", ins, offset_bytes=4)
+    assert e.value.code == "UNALIGNED"
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[8], "simple_ring", ins, offset_bytes=8)      # 16-byte messages
+    assert e.value.code == "UNALIGNED"
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[8], "simple", [a[:4 * 8 + 4] for a in ins])
+    assert e.value.code == "UNEVEN"
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[2], "bisect", ins[:2])
+    assert e.value.code == "TOPOLOGY"
+    with pytest.raises(vr.VRError) as e:
+        H.run_allreduce(ctxs[16], "simple", H.make_inputs(oracle, 16, 1 << 12, 3))
+    assert e.value.code == "TOPOLOGY"
+    # empty input: the reference's loop simply does not execute
+    empty = [np.zeros(0, np.uint16) for _ in range(8)]
+    got, _ = H.run_allreduce(ctxs[8], "simple", empty)
+    assert all(len(g) == 0 for g in got)
+
+
+def test_partial_overlap_is_rejected(ctxs):
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    big = DeviceBuffer(1 << 20)
+    n = 1 << 12
+    bufs = [big.ptr + r * n * 2 for r in range(8)]
+    outs = [big.ptr + r * n * 2 + 64 for r in range(8)]
+    with pytest.raises(vr.VRError) as e:
+        ctxs[8].allreduce("simple", bufs, n, outs=outs)
+    assert e.value.code == "OVERLAP"
+    big.free()
+
+
+def test_special_values(ctxs, oracle):
+    """Subnormals are kept, overflow goes to infinity, inf-inf gives NaN."""
+    rng = np.random.default_rng(11)
+    n = 8 * 4096
+    ins = []
+    for r in range(8):
+        a = rng.integers(0, 0x10000, n, dtype=np.uint32).astype(np.uint16)
+        a[(a & 0x7C00) == 0x7C00] &= 0x83FF           # finite inputs, every exponent
+        ins.append(a)
+    ins[0][:64] = 0x0001                               # smallest subnormals
+    ins[1][:64] = 0x8001
+    ins[2][64:128] = 0x7BFF                            # +max
+    ins[3][64:128] = 0x7BFF
+    ins[4][128:192] = 0x7C00                           # +inf and -inf
+    ins[5][128:192] = 0xFC00
+    for algo in ("simple", "bisect"):
+        got, _ = H.run_allreduce(ctxs[8], algo, ins)
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), algo)
+
+
+# ---- BASELINE configurations at full size ------------------------------------------------------
+
+def test_config1_two_ranks_simple(ctxs, oracle):
+    ins = H.make_inputs(oracle, 2, 16384, 1234, DIST_UNIFORM, -1.0, 1.0)
+    got, _ = H.run_allreduce(ctxs[2], "simple", ins, inplace=False)
+    want = oracle.rotated(ins)
+    assert (want == oracle.rank_order(ins)).all()      # N=2: every order coincides
+    H.assert_all_ranks_equal(oracle, got, want)
+
+
+def test_config2_small_1mib(ctxs, oracle):
+    ins = H.make_inputs(oracle, 8, 524288, 2000, DIST_NORMAL, 0.0, 1.0)
+    got, _ = H.run_allreduce(ctxs[8], "small", ins)
+    H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins))
+
+
+def test_config3_bisect_32mib(ctxs, oracle):
+    ins = H.make_inputs(oracle, 8, 16777216, 3000, DIST_NORMAL, 0.0, 0.02)
+    want = oracle.bisect(ins)
+    got, _ = H.run_allreduce(ctxs[8], "bisect", ins)
+    H.assert_all_ranks_equal(oracle, got, want)
+    assert oracle.count_mismatch(want, oracle.rotated(ins)) > 1000   # the tree really differs
+
+
+def test_config5_sweep_sizes(ctxs, oracle):
+    """4 KiB ... 256 MiB per rank in powers of two; the largest sizes are checked
+    on one protocol each to keep host memory and time bounded."""
+    for p in range(11, 28):
+        n = 1 << p
+        algos = ("small", "simple", "bisect") if p <= 22 else (("simple",) if p % 2 else ("bisect",))
+        ins = H.make_inputs(oracle, 8, n, 5000 + p)
+        for algo in algos:
+            got, _ = H.run_allreduce(ctxs[8], algo, ins)
+            want = H.expected(oracle, algo, ins)
+            # all ranks hold the same bits; compare rank 0 fully and the rest by equality
+            assert oracle.count_mismatch(got[0], want) == 0, (algo, n)
+            for r in range(1, 8):
+                assert oracle.count_mismatch(got[r], got[0]) == 0, (algo, n, r)
+
+
+# ---- all-gather ---------------------------------------------------------------------------------
+
+def run_allgather(ctx, algo, ins, alias_own_slot=False):
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    N, n = ctx.nranks, len(ins[0])
+    outs = [DeviceBuffer(N * n * 2 + 64) for _ in range(N)]
+    for o in outs:
+        o.fill(0x01)                                   # main.cpp:300 memsets the output to 1
+    if alias_own_slot:
+        in_ptrs = [outs[r].ptr + r * n * 2 for r in range(N)]
+        for r in range(N):
+            outs[r].upload(ins[r], r * n * 2)
+        srcs = []
+    else:
+        srcs = [DeviceBuffer(n * 2 + 64) for _ in range(N)]
+        for s, a in zip(srcs, ins):
+            s.upload(a)
+        in_ptrs = [s.ptr for s in srcs]
+    ctx.allgather(algo, in_ptrs, [o.ptr for o in outs], n)
+    ctx.check()
+    got = [o.download(np.uint16, N * n) for o in outs]
+    for b in outs + srcs:
+        b.free()
+    return got
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_allgather(ctxs, oracle, nranks, algo):
+    for n in (8, 8 * 15, 8 * 1237, 1 << 16):
+        ins = H.make_inputs(oracle, nranks, n, 70 + n, DIST_UNIFORM, -2.0, 2.0)
+        want = oracle.allgather(ins)
+        for alias in (False, True):
+            got = run_allgather(ctxs[nranks], algo, ins, alias)
+            for r in range(nranks):
+                assert (got[r] == want).all(), (n, r, alias)
+
+
+def test_config4_allgather_8mib(ctxs, oracle):
+    ins = H.make_inputs(oracle, 4, 4194304, 4000, DIST_UNIFORM, -2.0, 2.0)
+    want = oracle.allgather(ins)
+    got = run_allgather(ctxs[4], "allgather_simple", ins)
+    for r in range(4):
+        assert (got[r] == want).all()
+
+
+def test_allgather_rejections(ctxs, oracle):
+    ins = H.make_inputs(oracle, 4, 12, 1)                # 24 bytes: not a whole 16-byte message
+    with pytest.raises(vr.VRError) as e:
+        run_allgather(ctxs[4], "allgather_small", ins)
+    assert e.value.code == "UNEVEN"
