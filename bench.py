@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the single-shot all-reduce data path on one MI355X.
+
+A "step" is one all-reduce over the virtual ranks' buffers (already resident in
+HBM).  Default workload: 8 virtual ranks, `bisect`, 16,777,216 binary16 values
+(32 MiB) per rank, N(0, 0.02) inputs — the bandwidth-bound headline
+configuration.  Prints ONE JSON line; see --help for the other modes.
+
+Algorithmic bytes per step: B = N*S (every rank's input read once) + N*S (the sum
+written once to every rank's output) = 2*N*S.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (each scaled by the same counter's reading for a plain copy of known size);
+# see profiles/.  Keyed by workload name.
+MEASURED_TRAFFIC_BYTES = {}
+
+WORKLOADS = {
+    # name: (nranks, algo, nelems per rank, dist, p0, p1, seed)
+    "cfg2": (8, "small", 524288, 1, 0.0, 1.0, 2000),
+    "cfg3": (8, "bisect", 16777216, 1, 0.0, 0.02, 3000),
+    "cfg4": (4, "allgather_simple", 4194304, 0, -2.0, 2.0, 4000),
+}
+
+
+def describe(name):
+    n, algo, ne, dist, p0, p1, _ = WORKLOADS[name]
+    d = ("N(%g,%g)" % (p0, p1)) if dist == 1 else ("U[%g,%g)" % (p0, p1))
+    return "%s: %d virtual ranks, %s, %d binary16/rank (%.3g MiB), %s" % (
+        name, n, algo, ne, ne * 2 / 2**20, d)
+
+
+def algorithmic_bytes(name):
+    n, algo, ne, *_ = WORKLOADS[name]
+    s = ne * 2
+    if algo.startswith("allgather"):
+        return n * s + n * n * s
+    return 2 * n * s
+
+
+def setup(vr, binding, name, inplace, nsets=1):
+    """Context + `nsets` independent sets of per-rank device buffers holding the
+    same seeded inputs.  Rotating through several sets defeats the 256 MiB
+    memory-side cache, so that every step really streams from and to HBM."""
+    n, algo, ne, dist, p0, p1, seed = WORKLOADS[name]
+    ctx = vr.VirtualRanks(n)
+    host = [binding.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
+    sets = []
+    for _ in range(nsets):
+        ins = [binding.DeviceBuffer(ne * 2) for _ in range(n)]
+        for b, a in zip(ins, host):
+            b.upload(a)
+        if algo.startswith("allgather"):
+            outs = [binding.DeviceBuffer(n * ne * 2) for _ in range(n)]
+        elif inplace:
+            outs = None
+        else:
+            outs = [binding.DeviceBuffer(ne * 2) for _ in range(n)]
+        sets.append((ins, outs))
+    return ctx, host, sets
+
+
+def launch(ctx, name, ins, outs):
+    n, algo, ne, *_ = WORKLOADS[name]
+    if algo.startswith("allgather"):
+        ctx.allgather(algo, [b.ptr for b in ins], [b.ptr for b in outs], ne)
+    else:
+        ctx.allreduce(algo, [b.ptr for b in ins], ne, outs=[b.ptr for b in outs] if outs else None)
+
+
+def time_kernels(binding, ctx, name, sets, iters, group=1):
+    """Kernel times (ms per launch) from HIP event pairs recorded on the launch
+    stream, rotating through the buffer sets.  With group > 1 each pair brackets
+    `group` back-to-back launches and the result is their mean, which amortises
+    the ~2 us the event commands themselves add."""
+    npairs = (iters + group - 1) // group
+    timer = binding.EventTimer(npairs)
+    k = 0
+    for p in range(npairs):
+        timer.start(p)
+        for _ in range(group):
+            launch(ctx, name, *sets[k % len(sets)])
+            k += 1
+        timer.stop(p)
+    ctx.sync()
+    out = timer.elapsed_ms(npairs) / group
+    timer.close()
+    return out
+
+
+def hbm_ceilings(binding, ctx):
+    """Plain streaming kernels over 2 GiB (nothing cache-resident): what this
+    GPU's HBM delivers for pure reads, pure writes and a 1:1 copy."""
+    nbytes = 512 << 20
+    bufs = [binding.DeviceBuffer(nbytes) for _ in range(8)]
+    for b in bufs:
+        b.fill(0)
+    out = {}
+    for label, mode, moved in (("copy", 0, 2 * nbytes), ("read_only", 1, nbytes),
+                               ("write_only", 2, nbytes)):
+        timer = binding.EventTimer(24)
+        for k in range(24):       # src/dst walk over all eight buffers
+            timer.start(k)
+            ctx.stream_probe(mode, bufs[(2 * k + 1) % 8].ptr, bufs[(2 * k) % 8].ptr, nbytes)
+            timer.stop(k)
+        ctx.sync()
+        ms = timer.elapsed_ms()[8:]
+        timer.close()
+        out[label + "_GBps"] = round(moved / (float(np.median(ms)) * 1e-3) / 1e9, 1)
+    for b in bufs:
+        b.free()
+    return out
+
+
+def verify(name, host, ins, outs):
+    """Bit-exact check of the buffers against the CPU oracle (checker only)."""
+    from tests import oracle_lib
+    o = oracle_lib.load()
+    n, algo, ne, *_ = WORKLOADS[name]
+    if algo.startswith("allgather"):
+        want = o.allgather(host)
+    elif algo == "bisect":
+        want = o.bisect(host)
+    else:
+        want = o.rotated(host)
+    bad = 0
+    for b in (outs if outs else ins):
+        bad += o.count_mismatch(b.download(np.uint16, len(want)), want)
+    return bad
+
+
+def cpu_baseline(name, budget_s):
+    """The oracle's OpenMP loop for this workload on the host cores (reported only)."""
+    from tests import oracle_lib
+    o = oracle_lib.load()
+    n, algo, ne, dist, p0, p1, seed = WORKLOADS[name]
+    host = [o.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
+    fn = o.allgather if algo.startswith("allgather") else (o.bisect if algo == "bisect" else o.rotated)
+    out = {}
+    for label, threads in (("all", 0), ("one", 1)):
+        used = o.set_threads(threads if threads else (os.cpu_count() or 1))
+        if threads == 0:
+            env = os.environ.get("OMP_NUM_THREADS")
+            used = o.set_threads(int(env) if env else min(os.cpu_count() or 1, 64))
+        fn(host)                                          # warm-up, page faults
+        best, reps, t_start = 1e30, 0, time.perf_counter()
+        while True:
+            t0 = time.perf_counter()
+            fn(host)
+            dt = time.perf_counter() - t0
+            best, reps = min(best, dt), reps + 1
+            if reps >= 5 and time.perf_counter() - t_start > budget_s / 2:
+                break
+            if time.perf_counter() - t_start > budget_s:
+                break
+        out[label] = (algorithmic_bytes(name) / best / 1e9, used, reps, best)
+    gb_all, cores, reps, best = out["all"]
+    return {
+        "value": round(gb_all, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": "%s full size, best of %d passes (%.1f ms); 1 thread: %.3f GB/s" % (
+            name, reps, best * 1e3, out["one"][0]),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--inplace", action="store_true",
+                    help="reference semantics: results overwrite the inputs (values saturate "
+                         "after a few steps; traffic is identical)")
+    ap.add_argument("--sets", type=int, default=4,
+                    help="buffer sets the steps rotate through (1 = reuse one set, cache-warm)")
+    ap.add_argument("--event-group", type=int, default=10,
+                    help="launches bracketed by one HIP event pair when timing kernels")
+    ap.add_argument("--only-headline", action="store_true",
+                    help="run nothing but the headline workload (for profiler runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--latency-iters", type=int, default=1000)
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VAL")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every virtual rank lives in one MI355X's HBM; "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import gpu_ipc_example_amd as vr
+    from gpu_ipc_example_amd import binding
+
+    name = args.workload
+    n, algo, ne, *_ = WORKLOADS[name]
+    B = algorithmic_bytes(name)
+    ctx, host, sets = setup(vr, binding, name, args.inplace, args.sets)
+    for kv in args.tune:
+        k, v = kv.split("=")
+        ctx.set_tuning(**{k: int(v)})
+
+    # correctness of exactly this configuration, on fresh inputs
+    launch(ctx, name, *sets[0])
+    ctx.sync()
+    mismatches = verify(name, host, *sets[0])
+    if args.inplace:
+        for b, a in zip(sets[0][0], host):
+            b.upload(a)
+
+    for i in range(args.warmup):
+        launch(ctx, name, *sets[i % len(sets)])
+    ctx.sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        launch(ctx, name, *sets[i % len(sets)])
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = B / (wall / args.steps) / 1e9
+
+    # kernel durations of the same K launches, from HIP events on the launch stream
+    kms = time_kernels(binding, ctx, name, sets, args.steps, group=args.event_group)
+    k_avg = float(kms.mean())
+    achieved = B / (k_avg * 1e-3) / 1e9
+
+    result = {
+        "metric": "allreduce_algorithmic_hbm_bandwidth_8vrank_fp16_32MiB_per_rank"
+                  if name == "cfg3" else "algorithmic_hbm_bandwidth_" + name,
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": describe(name), "virtual_ranks": n, "protocol": algo,
+                   "bytes_per_rank": ne * 2, "in_place": bool(args.inplace),
+                   "algorithmic_bytes_per_step": B, "buffer_sets_rotated": len(sets),
+                   "note": "steps rotate through %d buffer sets (%.0f MiB touched) so the 256 MiB "
+                           "memory-side cache cannot serve them" % (
+                               len(sets), len(sets) * (B if not args.inplace else B / 2) / 2**20)
+                           if len(sets) > 1 else "every step reuses one buffer set (cache-warm)"},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "bit_exact_vs_oracle": mismatches == 0, "mismatches": int(mismatches),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "kernel_us_avg": round(k_avg * 1e3, 3),
+                     "kernel_us_p50": round(float(np.median(kms)) * 1e3, 3)},
+    }
+    if not algo.startswith("allgather"):
+        strict = (n + 1) * ne * 2
+        result["strict_GBps_(N+1)S"] = round(strict / (k_avg * 1e-3) / 1e9, 2)
+
+    if len(sets) > 1 and not args.only_headline:
+        # the same launches on ONE buffer set: inputs stay in the memory-side cache
+        time_kernels(binding, ctx, name, sets[:1], 10)
+        wms = time_kernels(binding, ctx, name, sets[:1], 50, group=10)
+        result["same_buffers_cache_warm"] = {
+            "GBps": round(B / (float(wms.mean()) * 1e-3) / 1e9, 2),
+            "kernel_us_avg": round(float(wms.mean()) * 1e3, 3),
+            "note": "Infinity-Cache assisted; not an HBM figure"}
+
+    if name == "cfg3" and not args.only_headline:
+        # second half of the metric: p50 latency of the 1 MiB/rank `small` all-reduce
+        c2, h2, s2 = setup(vr, binding, "cfg2", True, 1)
+        launch(c2, "cfg2", *s2[0])
+        c2.sync()
+        bad2 = verify("cfg2", h2, *s2[0])
+        time_kernels(binding, c2, "cfg2", s2, 50)
+        lat = time_kernels(binding, c2, "cfg2", s2, args.latency_iters) * 1e3
+        p50 = float(np.percentile(lat, 50))
+        result["latency_1MiB_per_rank"] = {
+            "workload": describe("cfg2") + ", in place", "iters": args.latency_iters,
+            "p50_us": round(p50, 3), "p99_us": round(float(np.percentile(lat, 99)), 3),
+            "min_us": round(float(lat.min()), 3), "bit_exact_vs_oracle": bad2 == 0,
+            "GBps_at_p50": round(algorithmic_bytes("cfg2") / (p50 * 1e-6) / 1e9, 1),
+            "note": "one HIP event pair per launch: includes ~2 us of event overhead that a "
+                    "kernel trace does not show; buffers are cache-resident"}
+        result["hbm_ceilings"] = hbm_ceilings(binding, ctx)
+
+    if not args.no_cpu and not args.only_headline:
+        result["cpu_baseline"] = cpu_baseline(name, args.cpu_seconds)
+    print(json.dumps(result, default=float))
+
+
+if __name__ == "__main__":
+    main()

@@ -84,6 +84,7 @@ def lib():
         "vr_time_allreduce": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_copy": (i, [vp, vp, vp, vp, sz, i, C.POINTER(C.c_float)]),
+        "vr_stream_probe": (i, [vp, vp, i, vp, vp, sz]),
         "vr_fill_pattern": (None, [C.POINTER(C.c_uint16), i, sz]),
         "vr_generate": (None, [C.POINTER(C.c_uint16), sz, C.c_uint64, i, C.c_double, C.c_double]),
         "vr_parse_nelems": (i, [C.c_char_p, C.POINTER(sz)]),
@@ -97,6 +98,10 @@ def lib():
         "vr_stream_create": (i, [i, vpp]),
         "vr_stream_destroy": (i, [vp]),
         "vr_stream_sync": (i, [vp]),
+        "vr_event_create": (i, [vpp]),
+        "vr_event_record": (i, [vp, vp]),
+        "vr_event_elapsed_ms": (i, [vp, vp, C.POINTER(C.c_float)]),
+        "vr_event_destroy": (i, [vp]),
         "vr_strerror": (C.c_char_p, [i]),
         "vr_last_error_detail": (C.c_char_p, []),
         "vr_version": (C.c_char_p, []),
@@ -273,8 +278,44 @@ class VirtualRanks:
                                        _table(outputs), nelems, iters, ms))
         return np.frombuffer(ms, np.float32).copy()
 
+    def stream_probe(self, mode, dst, src, nbytes, stream=None):
+        """mode: 0 copy, 1 read only, 2 write only."""
+        _check(lib().vr_stream_probe(self._h, stream, mode, C.c_void_p(int(dst)),
+                                     C.c_void_p(int(src)), nbytes))
+
     def time_copy(self, dst, src, nbytes, iters, stream=None):
         ms = (C.c_float * iters)()
         _check(lib().vr_time_copy(self._h, stream, C.c_void_p(int(dst)), C.c_void_p(int(src)), nbytes,
                                   iters, ms))
         return np.frombuffer(ms, np.float32).copy()
+
+
+class EventTimer:
+    """Pairs of HIP events recorded on one stream around caller-chosen launches."""
+
+    def __init__(self, pairs, stream=None):
+        self.stream, self.events = stream, []
+        for _ in range(2 * pairs):
+            e = C.c_void_p()
+            _check(lib().vr_event_create(C.byref(e)))
+            self.events.append(e)
+
+    def start(self, k):
+        _check(lib().vr_event_record(self.events[2 * k], self.stream))
+
+    def stop(self, k):
+        _check(lib().vr_event_record(self.events[2 * k + 1], self.stream))
+
+    def elapsed_ms(self, count=None):
+        count = len(self.events) // 2 if count is None else count
+        out = np.empty(count, np.float32)
+        ms = C.c_float(0)
+        for k in range(count):
+            _check(lib().vr_event_elapsed_ms(self.events[2 * k], self.events[2 * k + 1], C.byref(ms)))
+            out[k] = ms.value
+        return out
+
+    def close(self):
+        for e in self.events:
+            lib().vr_event_destroy(e)
+        self.events = []

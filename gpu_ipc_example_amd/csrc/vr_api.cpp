@@ -194,11 +194,15 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 // context
 // ---------------------------------------------------------------------------------
 
+// User overrides of the launch heuristics; -1 = let the library decide.
+struct TuningOverrides {
+  int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
+};
+
 struct vr_ctx {
   int nranks = 0;
   DeviceInfo dev;
-  Tuning tuning;
-  bool tuning_user_block = false;
+  TuningOverrides tune;
   uint32_t seq_no = 1;
   uint64_t spin_limit = 0;
 };
@@ -244,24 +248,29 @@ extern "C" int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls) {
 
 static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!ctx || !key) return nullptr;
-  if (!strcmp(key, "block")) return &ctx->tuning.block;
-  if (!strcmp(key, "waves_per_cu")) return &ctx->tuning.waves_per_cu;
-  if (!strcmp(key, "unroll")) return &ctx->tuning.unroll;
-  if (!strcmp(key, "nt_load")) return &ctx->tuning.nt_load;
-  if (!strcmp(key, "nt_store")) return &ctx->tuning.nt_store;
-  if (!strcmp(key, "oneshot")) return &ctx->tuning.oneshot;
+  if (!strcmp(key, "block")) return &ctx->tune.block;
+  if (!strcmp(key, "waves_per_cu")) return &ctx->tune.waves_per_cu;
+  if (!strcmp(key, "unroll")) return &ctx->tune.unroll;
+  if (!strcmp(key, "nt_load")) return &ctx->tune.nt_load;
+  if (!strcmp(key, "nt_store")) return &ctx->tune.nt_store;
+  if (!strcmp(key, "oneshot")) return &ctx->tune.oneshot;
   return nullptr;
 }
 
 extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
   int *f = tuning_field(ctx, key);
   if (!f) return fail(VR_ERR_INVALID, std::string("unknown tuning key ") + (key ? key : "(null)"));
-  if (!strcmp(key, "block") && (value < 64 || value > 1024 || value % 64))
-    return fail(VR_ERR_INVALID, "block must be a multiple of 64 in [64,1024]");
-  if (!strcmp(key, "waves_per_cu") && (value < 1 || value > 64))
-    return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
-  if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
-    return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
+  if (value != -1) {
+    if (!strcmp(key, "block") && (value < 64 || value > 1024 || value % 64))
+      return fail(VR_ERR_INVALID, "block must be a multiple of 64 in [64,1024]");
+    if (!strcmp(key, "waves_per_cu") && (value < 1 || value > 64))
+      return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
+    if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
+      return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "nt_store") || !strcmp(key, "oneshot")) &&
+        !(value == 0 || value == 1))
+      return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
+  }
   *f = value;
   return VR_OK;
 }
@@ -283,17 +292,43 @@ static bool ranges_partially_overlap(const void *a, const void *b, size_t bytes)
   return x < y + bytes && y < x + bytes;
 }
 
-static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a) {
-  Tuning t = ctx->tuning;
+// Launch heuristics of the direct kernels.  `read_bytes` / `write_bytes` are the
+// distinct bytes a launch reads and writes; what matters is how they compare with
+// the 256 MiB memory-side cache (Infinity Cache) in front of HBM.
+static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes, size_t write_bytes,
+                         bool in_place) {
+  const size_t kMall = 256ull << 20;
+  Tuning t;
+  t.block = 256;
+  t.waves_per_cu = 8;
+  t.unroll = 1;
   if (a->latency_tuned) {
-    // "small" family: every lane makes one trip, results stay cacheable for
-    // the kernel that consumes them next.
+    // "small" family: every lane makes one trip; results stay cacheable for the
+    // kernel that consumes them next.
     t.oneshot = 1;
-    t.unroll = 1;
     t.nt_load = 0;
     t.nt_store = 0;
-    t.block = 256;
+  } else {
+    t.oneshot = 0;
+    const size_t footprint = in_place ? read_bytes : read_bytes + write_bytes;
+    if (footprint <= kMall) {            // everything can live in the memory-side cache
+      t.nt_load = 0;
+      t.nt_store = 0;
+    } else if (read_bytes <= kMall) {    // keep the inputs cacheable, stream the results past them
+      t.nt_load = 0;
+      t.nt_store = 1;
+    } else {                             // pure streaming
+      t.nt_load = 1;
+      t.nt_store = 1;
+    }
   }
+  const TuningOverrides &o = ctx->tune;
+  if (o.block != -1) t.block = o.block;
+  if (o.waves_per_cu != -1) t.waves_per_cu = o.waves_per_cu;
+  if (o.unroll != -1) t.unroll = o.unroll;
+  if (o.nt_load != -1) t.nt_load = o.nt_load;
+  if (o.nt_store != -1) t.nt_store = o.nt_store;
+  if (o.oneshot != -1) t.oneshot = o.oneshot;
   return t;
 }
 
@@ -303,6 +338,8 @@ struct Prepared {
   size_t chunk_elems;
   int vec_halves;
   vr_geometry geom;
+  bool in_place;
+  size_t bytes_all_ranks;   // nranks * nelems * 2
 };
 
 static int prepare_allreduce(vr_ctx *ctx, int algo, void *const bufs[], void *const outs[],
@@ -334,6 +371,9 @@ static int prepare_allreduce(vr_ctx *ctx, int algo, void *const bufs[], void *co
   }
   p->chunk_elems = work / 2;
   p->vec_halves = (align16 && p->chunk_elems % 8 == 0) ? 8 : 4;
+  p->in_place = true;
+  for (int r = 0; r < N; ++r) p->in_place = p->in_place && (p->in.p[r] == p->out.p[r]);
+  p->bytes_all_ranks = (size_t)N * nelems * 2;
   return vr_launch_geometry(algo, N, nelems, &p->geom);
 }
 
@@ -365,7 +405,7 @@ extern "C" int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, 
   if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
   const uint32_t start = *seq;
-  if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr, tuning_for(ctx, p.a), start)) return rc;
+  if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr, tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place), start)) return rc;
   *seq = start + p.geom.steps;   // getLaunchParam: updateSeqNo += nSteps
   return VR_OK;
 }
@@ -385,7 +425,7 @@ extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transp
   // Map the reference's (groups x subgroups x simd) grid onto wavefronts: a block
   // holds the same number of lanes (rounded to whole waves, at most 1024) and the
   // launch holds ceil(groups / nranks) blocks for every virtual rank.
-  Tuning t = ctx->tuning;
+  Tuning t = tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place);
   size_t lanes = (size_t)subgroups * simd;
   lanes = ((lanes + 63) / 64) * 64;
   if (lanes > 1024) lanes = 1024;
@@ -445,7 +485,9 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
   if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
   if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
-  hipError_t e = launch_direct_allgather((hipStream_t)stream, ctx->dev, tuning_for(ctx, p.a),
+  const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
+  hipError_t e = launch_direct_allgather((hipStream_t)stream, ctx->dev,
+                                         tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false),
                                          ctx->nranks, p.in, p.out, nelems, p.vec_halves);
   if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
@@ -498,7 +540,7 @@ extern "C" int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transp
   if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
   int tr;
   if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
-  const Tuning t = tuning_for(ctx, p.a);
+  const Tuning t = tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place);
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
     const uint32_t start = ctx->seq_no;
@@ -514,7 +556,8 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   PreparedGather p;
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
   if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
-  const Tuning t = tuning_for(ctx, p.a);
+  const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
+  const Tuning t = tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false);
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
     hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);
@@ -522,13 +565,44 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   });
 }
 
+// The probes are pure streaming: nontemporal both ways, large blocks, four
+// 16-byte vectors per lane in flight (what measured best for a plain copy).
+static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, Tuning *t) {
+  if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
+  if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16)
+    return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
+  Tuning d;
+  d.block = 1024;
+  d.waves_per_cu = 16;
+  d.unroll = 4;
+  d.nt_load = d.nt_store = 1;
+  d.oneshot = 0;
+  const TuningOverrides &o = ctx->tune;
+  if (o.block != -1) d.block = o.block;
+  if (o.waves_per_cu != -1) d.waves_per_cu = o.waves_per_cu;
+  if (o.unroll != -1) d.unroll = o.unroll;
+  if (o.nt_load != -1) d.nt_load = o.nt_load;
+  if (o.nt_store != -1) d.nt_store = o.nt_store;
+  *t = d;
+  return VR_OK;
+}
+
+extern "C" int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, const void *src,
+                               size_t bytes) {
+  Tuning t;
+  if (mode < 0 || mode > 2) return fail(VR_ERR_INVALID, "bad probe mode");
+  if (int rc = copy_tuning(ctx, dst, src, bytes, &t)) return rc;
+  hipError_t e = launch_copy((hipStream_t)stream, ctx->dev, t, dst, src, bytes, mode);
+  return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
+}
+
 extern "C" int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes,
                             int iters, float *ms_out) {
-  if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
-  if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16) return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
+  Tuning t;
+  if (int rc = copy_tuning(ctx, dst, src, bytes, &t)) return rc;
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
-    hipError_t e = launch_copy(s, ctx->dev, ctx->tuning, dst, src, bytes);
+    hipError_t e = launch_copy(s, ctx->dev, t, dst, src, bytes);
     return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
   });
 }
@@ -657,5 +731,30 @@ extern "C" int vr_stream_destroy(void *stream) {
 
 extern "C" int vr_stream_sync(void *stream) {
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return VR_OK;
+}
+
+extern "C" int vr_event_create(void **event_out) {
+  if (!event_out) return fail(VR_ERR_INVALID, "null argument");
+  hipEvent_t e;
+  HIP_TRY(hipEventCreate(&e));
+  *event_out = e;
+  return VR_OK;
+}
+
+extern "C" int vr_event_record(void *event, void *stream) {
+  HIP_TRY(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+  return VR_OK;
+}
+
+extern "C" int vr_event_elapsed_ms(void *start, void *stop, float *ms_out) {
+  if (!ms_out) return fail(VR_ERR_INVALID, "null argument");
+  HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+  HIP_TRY(hipEventElapsedTime(ms_out, (hipEvent_t)start, (hipEvent_t)stop));
+  return VR_OK;
+}
+
+extern "C" int vr_event_destroy(void *event) {
+  if (event) HIP_TRY(hipEventDestroy((hipEvent_t)event));
   return VR_OK;
 }

@@ -177,21 +177,40 @@ __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable
   }
 }
 
-template <int UNROLL, bool NT_LD, bool NT_ST>
-__global__ __launch_bounds__(1024) void k_copy(h8 *dst, const h8 *src, size_t vecs) {
+// Streaming yardsticks: MODE 0 copies, 1 only reads (the sum is kept alive by a
+// store that never executes for finite data), 2 only writes.
+template <int MODE, int UNROLL, bool NT>
+__global__ __launch_bounds__(1024) void k_probe(h8 *dst, const h8 *src, size_t vecs) {
   const size_t tile = (size_t)blockDim.x * UNROLL;
   const size_t stride = tile * gridDim.x;
+  h8 acc = {0, 0, 0, 0, 0, 0, 0, 0};
   for (size_t base = (size_t)blockIdx.x * tile; base < vecs; base += stride) {
-    h8 x[UNROLL];
-    size_t idx[UNROLL];
+    const size_t first = base + threadIdx.x;
+    if (base + tile <= vecs) {
+      h8 x[UNROLL];
+      if constexpr (MODE != 2) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      idx[u] = base + (size_t)u * blockDim.x + threadIdx.x;
-      if (idx[u] < vecs) x[u] = ld<h8, NT_LD>(src + idx[u]);
+        for (int u = 0; u < UNROLL; ++u) x[u] = ld<h8, NT>(src + first + (size_t)u * blockDim.x);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        if constexpr (MODE == 0) st<h8, NT>(dst + first + (size_t)u * blockDim.x, x[u]);
+        if constexpr (MODE == 1) acc = acc + x[u];
+        if constexpr (MODE == 2) st<h8, NT>(dst + first + (size_t)u * blockDim.x, acc);
+      }
+    } else {
+      for (int u = 0; u < UNROLL; ++u) {
+        const size_t i = first + (size_t)u * blockDim.x;
+        if (i < vecs) {
+          if constexpr (MODE == 0) st<h8, NT>(dst + i, ld<h8, NT>(src + i));
+          if constexpr (MODE == 1) acc = acc + ld<h8, NT>(src + i);
+          if constexpr (MODE == 2) st<h8, NT>(dst + i, acc);
+        }
+      }
     }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-      if (idx[u] < vecs) st<h8, NT_ST>(dst + idx[u], x[u]);
+  }
+  if constexpr (MODE == 1) {
+    if (acc[0] == (_Float16)12345.0f && acc[7] == (_Float16)-321.0f) dst[0] = acc;
   }
 }
 
@@ -323,10 +342,10 @@ hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const T
 }
 
 hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, void *dst,
-                       const void *src, size_t bytes) {
+                       const void *src, size_t bytes, int mode) {
   const size_t vecs = bytes / 16;
   if (vecs == 0) return hipSuccess;
-  const int unroll = t.unroll >= 4 ? 4 : (t.unroll >= 2 ? 2 : 1);
+  const int unroll = t.unroll >= 4 ? 4 : 1;
   const size_t tile = (size_t)t.block * unroll;
   size_t blocks = (vecs + tile - 1) / tile;
   const size_t resident = (size_t)dev.cus * t.waves_per_cu / (t.block / 64);
@@ -334,23 +353,26 @@ hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, vo
   const dim3 grid((uint32_t)blocks), block(t.block);
   h8 *d = static_cast<h8 *>(dst);
   const h8 *sp = static_cast<const h8 *>(src);
-#define VR_COPY(U)                                                                          \
-  if (t.nt_load && t.nt_store)                                                              \
-    hipLaunchKernelGGL((k_copy<U, true, true>), grid, block, 0, s, d, sp, vecs);             \
-  else if (t.nt_load)                                                                       \
-    hipLaunchKernelGGL((k_copy<U, true, false>), grid, block, 0, s, d, sp, vecs);            \
-  else if (t.nt_store)                                                                      \
-    hipLaunchKernelGGL((k_copy<U, false, true>), grid, block, 0, s, d, sp, vecs);            \
-  else                                                                                      \
-    hipLaunchKernelGGL((k_copy<U, false, false>), grid, block, 0, s, d, sp, vecs);
-  if (unroll == 4) {
-    VR_COPY(4)
-  } else if (unroll == 2) {
-    VR_COPY(2)
-  } else {
-    VR_COPY(1)
+#define VR_PROBE(M, U)                                                                    \
+  if (t.nt_load || t.nt_store)                                                            \
+    hipLaunchKernelGGL((k_probe<M, U, true>), grid, block, 0, s, d, sp, vecs);             \
+  else                                                                                    \
+    hipLaunchKernelGGL((k_probe<M, U, false>), grid, block, 0, s, d, sp, vecs);
+#define VR_PROBE_U(M)  \
+  if (unroll == 4) {   \
+    VR_PROBE(M, 4)     \
+  } else {             \
+    VR_PROBE(M, 1)     \
   }
-#undef VR_COPY
+  if (mode == 1) {
+    VR_PROBE_U(1)
+  } else if (mode == 2) {
+    VR_PROBE_U(2)
+  } else {
+    VR_PROBE_U(0)
+  }
+#undef VR_PROBE_U
+#undef VR_PROBE
   return hipGetLastError();
 }
 

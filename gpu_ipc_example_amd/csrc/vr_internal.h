@@ -46,7 +46,8 @@ hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const T
 hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
                                    const PtrTable &in, const PtrTable &out, size_t nelems,
                                    int vec_halves);
+// mode: 0 copy, 1 read only, 2 write only
 hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, void *dst,
-                       const void *src, size_t bytes);
+                       const void *src, size_t bytes, int mode = 0);
 
 }  // namespace vr

@@ -174,6 +174,13 @@ int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
  * same way: the practical HBM ceiling next to which the all-reduce is read. */
 int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes, int iters,
                  float *ms_out);
+/* One asynchronous launch of a plain streaming kernel over `bytes` (16-byte
+ * granules): the yardsticks an all-reduce figure is read against.
+ *   VR_PROBE_COPY  dst[i] = src[i]         (bytes read + bytes written)
+ *   VR_PROBE_READ  reads src, writes nothing
+ *   VR_PROBE_WRITE writes dst, reads nothing */
+enum { VR_PROBE_COPY = 0, VR_PROBE_READ = 1, VR_PROBE_WRITE = 2 };
+int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, const void *src, size_t bytes);
 
 /* ---- host helpers -------------------------------------------------------------- */
 
@@ -196,6 +203,11 @@ int vr_copy_to_host(void *dst_host, const void *src, size_t bytes);
 int vr_stream_create(int device, void **stream_out);
 int vr_stream_destroy(void *stream);
 int vr_stream_sync(void *stream);
+/* HIP events recorded on `stream`, for callers that time their own launch sequences. */
+int vr_event_create(void **event_out);
+int vr_event_record(void *event, void *stream);
+int vr_event_elapsed_ms(void *start, void *stop, float *ms_out);   /* waits for `stop` */
+int vr_event_destroy(void *event);
 
 /* ---- errors ---------------------------------------------------------------------- */
 
