@@ -1,0 +1,209 @@
+// vr_main — command-line harness of the virtual-rank all-reduce, with the flags
+// and the run protocol of the reference's main.cpp:
+//   -n/--nelems "8MB"  elements per rank, K/M/G suffix = x1024     (main.cpp:17-34, 177)
+//   -g/--groups, -w/--subgroups, -s/--simd   launch grid           (main.cpp:179-187, 289-294)
+//   -f/--flag          first sequence number (default 0xe00f100f)  (main.cpp:183)
+//   -v/--verify        check run #1 against the host sum and stop  (main.cpp:75-84)
+//   -a/--algo          small | simple | bisect | ... | allgather_* (main.cpp:190, 296)
+// plus what one process driving all ranks needs:
+//   -r/--ranks N       number of virtual ranks (the MPI world size of the reference)
+//   -t/--transport     direct | wire
+//   -d/--device        HIP device index
+// Run protocol (main.cpp:48-109): run #1 with `flag`; with -v verify and return;
+// otherwise two more warm-ups (flag+100, flag+150), then the timed run (flag+200)
+// whose kernel time is printed as "[rank] Running time: <ns>ns" for every rank.
+// All runs are in place on the same inputs, exactly like the reference.
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "vrank/allreduce.hpp"
+
+namespace {
+
+struct Options {
+  std::string nelems = "8MB", algo = "small", transport = "default";
+  size_t groups = 1, subgroups = 4, flag = 0xe00f100f;
+  uint32_t simd = 16;
+  bool verify = false, grid_given = false;
+  int ranks = 8, device = 0;
+};
+
+bool take(int &i, int argc, char **argv, const char *s, const char *l, std::string *out) {
+  const std::string a = argv[i];
+  const std::string ls = std::string("--") + l, ss = std::string("-") + s;
+  if (a == ls || a == ss) {
+    if (i + 1 >= argc) throw std::invalid_argument("missing value for " + a);
+    *out = argv[++i];
+    return true;
+  }
+  if (a.rfind(ls + "=", 0) == 0) { *out = a.substr(ls.size() + 1); return true; }
+  if (a.rfind(ss, 0) == 0 && a.size() > 2 && a[1] != '-') { *out = a.substr(2); return true; }  // -g64
+  return false;
+}
+
+Options parse(int argc, char **argv) {
+  Options o;
+  for (int i = 1; i < argc; ++i) {
+    std::string v;
+    const std::string a = argv[i];
+    if (a == "-v" || a == "--verify") { o.verify = true; continue; }
+    if (a == "-h" || a == "--help") {
+      printf("usage: vr_main [-n 8MB] [-r 8] [-a small|simple|bisect|parallel|small_ring|simple_ring|"
+             "small_pcie|simple_pcie|small_pcie_p|simple_pcie_p|allgather_small|allgather_simple]\n"
+             "               [-g groups -w subgroups -s simd] [-f flag] [-t direct|wire] [-d device] [-v]\n");
+      exit(0);
+    }
+    if (take(i, argc, argv, "n", "nelems", &v)) o.nelems = v;
+    else if (take(i, argc, argv, "g", "groups", &v)) { o.groups = strtoull(v.c_str(), nullptr, 0); o.grid_given = true; }
+    else if (take(i, argc, argv, "w", "subgroups", &v)) { o.subgroups = strtoull(v.c_str(), nullptr, 0); o.grid_given = true; }
+    else if (take(i, argc, argv, "f", "flag", &v)) o.flag = strtoull(v.c_str(), nullptr, 0);
+    else if (take(i, argc, argv, "s", "simd", &v)) o.simd = (uint32_t)strtoul(v.c_str(), nullptr, 0);
+    else if (take(i, argc, argv, "a", "algo", &v)) o.algo = v;
+    else if (take(i, argc, argv, "r", "ranks", &v)) o.ranks = atoi(v.c_str());
+    else if (take(i, argc, argv, "t", "transport", &v)) o.transport = v;
+    else if (take(i, argc, argv, "d", "device", &v)) o.device = atoi(v.c_str());
+    // the reference ignores what it does not know (allow_unrecognised_options)
+  }
+  return o;
+}
+
+// Host-side binary16 sum in rank order, like allreduce.cpp:18-27 does on sycl::half.
+// _Float16 arithmetic rounds to nearest even at every assignment.
+uint16_t h_bits(_Float16 h) { uint16_t u; memcpy(&u, &h, 2); return u; }
+_Float16 h_from(uint16_t u) { _Float16 h; memcpy(&h, &u, 2); return h; }
+
+int verify_allreduce(const std::vector<std::vector<uint16_t>> &got, int world, size_t nelems) {
+  std::vector<std::vector<uint16_t>> ranks(world, std::vector<uint16_t>(nelems));
+  for (int r = 0; r < world; ++r) vr_fill_pattern(ranks[r].data(), r, nelems);
+  size_t printed = 0, bad = 0;
+  for (int rank = 0; rank < world; ++rank)
+    for (size_t i = 0; i < nelems; ++i) {
+      _Float16 sum = (_Float16)0.0f;
+      for (int r = 0; r < world; ++r) sum = (_Float16)(sum + h_from(ranks[r][i]));
+      if (h_bits(sum) != got[rank][i]) {
+        ++bad;
+        if (printed++ < 16)
+          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", (double)sum,
+                 (double)h_from(got[rank][i]), rank, i);
+      }
+    }
+  if (bad == 0) printf("verify: %d ranks x %zu elements match the host sum\n", world, nelems);
+  else printf("verify: %zu mismatches\n", bad);
+  return 0;   // the reference's verify never fails the process (allreduce.cpp:550)
+}
+
+int verify_allgather(const std::vector<std::vector<uint16_t>> &got, int world, size_t nelems) {
+  std::vector<uint16_t> want(nelems * world);
+  for (int r = 0; r < world; ++r) vr_fill_pattern(want.data() + (size_t)r * nelems, r, nelems);
+  size_t printed = 0, bad = 0;
+  for (int rank = 0; rank < world; ++rank)
+    for (size_t i = 0; i < nelems * world; ++i)
+      if (want[i] != got[rank][i]) {
+        ++bad;
+        if (printed++ < 16)
+          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", (double)h_from(want[i]),
+                 (double)h_from(got[rank][i]), rank, i);
+      }
+  if (bad == 0) printf("verify: %d ranks x %zu gathered elements match\n", world, nelems * world);
+  else printf("verify: %zu mismatches\n", bad);
+  return 0;
+}
+
+}  // namespace
+
+int main(int argc, char **argv) try {
+  const Options o = parse(argc, argv);
+  size_t nelems = 0;
+  vrank::check(vr_parse_nelems(o.nelems.c_str(), &nelems));
+  const int world = o.ranks;
+  const bool gather = o.algo.find("allgather") != std::string::npos;
+  int algo = -1;
+  vrank::check(vr_algo_from_string(o.algo.c_str(), &algo));
+
+  if (o.grid_given && o.subgroups % 4 != 0)
+    throw std::logic_error("Subgroup numbers must be multiple of 4");   // main.cpp:289-291
+
+  vrank::VirtualRanks ranks(world, o.device);
+  if (o.transport == "direct") ranks.setTransport(VR_TRANSPORT_DIRECT);
+  else if (o.transport == "wire") ranks.setTransport(VR_TRANSPORT_WIRE);
+  else if (o.transport != "default") throw std::invalid_argument("transport must be direct or wire");
+
+  const size_t alloc = nelems * sizeof(uint16_t);
+  std::vector<void *> input(world, nullptr), output(world, nullptr);
+  std::vector<uint16_t> host(nelems);
+  for (int r = 0; r < world; ++r) {
+    vrank::check(vr_malloc(o.device, alloc, &input[r]));
+    vr_fill_pattern(host.data(), r, nelems);
+    vrank::check(vr_copy_to_device(input[r], host.data(), alloc));
+    if (gather) {
+      vrank::check(vr_malloc(o.device, alloc * world, &output[r]));
+      vrank::check(vr_memset(output[r], 1, alloc * world));          // main.cpp:300
+    }
+  }
+  void *stream = nullptr;
+  vrank::check(vr_stream_create(o.device, &stream));
+  void *ev0 = nullptr, *ev1 = nullptr;
+  vrank::check(vr_event_create(&ev0));
+  vrank::check(vr_event_create(&ev1));
+
+  auto run = [&](uint32_t flag) {
+    uint32_t step = flag;
+    if (gather) {
+      vrank::check(vr_allgather(ranks.get(), stream, algo, ranks.transport(),
+                                (const void *const *)input.data(), output.data(), nelems, &step));
+    } else if (o.grid_given) {
+      vrank::check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transport(), input.data(),
+                                     nullptr, nelems, flag, (uint32_t)o.groups,
+                                     (uint32_t)o.subgroups, o.simd));
+    } else {
+      vrank::check(vr_allreduce(ranks.get(), stream, algo, ranks.transport(), input.data(), nullptr,
+                                nelems, &step));
+    }
+  };
+
+  run((uint32_t)o.flag);
+  ranks.wait(stream);
+
+  if (o.verify) {
+    std::vector<std::vector<uint16_t>> got(world);
+    for (int r = 0; r < world; ++r) {
+      got[r].resize(gather ? nelems * world : nelems);
+      vrank::check(vr_copy_to_host(got[r].data(), gather ? output[r] : input[r], got[r].size() * 2));
+    }
+    return gather ? verify_allgather(got, world, nelems) : verify_allreduce(got, world, nelems);
+  }
+
+  run((uint32_t)o.flag + 100);
+  run((uint32_t)o.flag + 150);
+  printf("---------last run------------------\n");
+  ranks.wait(stream);
+  vrank::check(vr_event_record(ev0, stream));
+  run((uint32_t)o.flag + 200);
+  vrank::check(vr_event_record(ev1, stream));
+  float ms = 0.f;
+  vrank::check(vr_event_elapsed_ms(ev0, ev1, &ms));
+  ranks.wait(stream);
+  for (int r = 0; r < world; ++r) printf("[%d] Running time: %lluns\n", r, (unsigned long long)(ms * 1e6));
+  const double bytes = gather ? (double)world * alloc + (double)world * world * alloc
+                              : 2.0 * world * alloc;
+  printf("%s: %d ranks x %zu halves, %.3f us, %.1f GB/s algorithmic (2*N*S%s)\n", o.algo.c_str(),
+         world, nelems, ms * 1e3, bytes / (ms * 1e-3) / 1e9, gather ? " -> N*S + N*N*S" : "");
+
+  vr_event_destroy(ev0);
+  vr_event_destroy(ev1);
+  vr_stream_destroy(stream);
+  for (int r = 0; r < world; ++r) {
+    vr_free(input[r]);
+    vr_free(output[r]);
+  }
+  return 0;
+} catch (const std::exception &e) {
+  fprintf(stderr, "vr_main: %s\n", e.what());
+  return 1;
+}

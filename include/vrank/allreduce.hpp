@@ -1,0 +1,337 @@
+// vrank/allreduce.hpp — C++ host API over the C ABI in vrank_allreduce.h.
+//
+// Mirrors the reference's host-side types so that code written against
+//   AllReduce<T, NRanks, Proto, Transmit, SubGroupSize>        (allreduce.hpp:8-28, 64-74)
+//   bisectPAllReduce<T, NRanks, Transmit, SubGroupSize>        (allreduce.hpp:212-270)
+//   AllGather<T, NRanks, Proto, Transmit, SubGroupSize>        (allgather.hpp:8-70)
+//   testTransmit<T>(std::string algo, ...) / testAllgather     (allreduce.cpp:1118-1213)
+// keeps its shape: construct, then launch on a stream; the protocol is chosen by
+// the <Proto, Transmit> template arguments or by the -a string.  What changes is
+// the meaning of "rank": the NRanks peers are virtual ranks, separate device
+// allocations inside one GPU, so one object drives all of them and the peer
+// scratch tables of the reference's constructor collapse into a VirtualRanks
+// handle.  Errors come back as the reference's std::logic_error texts.
+//
+// Header-only; needs nothing but the C ABI (no HIP headers).  A stream is passed
+// as void* (a hipStream_t).
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "../vrank_allreduce.h"
+
+namespace vrank {
+
+// ---- errors ---------------------------------------------------------------------
+// The reference throws std::logic_error for everything its host code rejects
+// (allreduce.hpp:110-118; allreduce.cpp:880, 917, 1187; main.cpp:290).  Runtime
+// failures that have no counterpart there (HIP errors, poll time-outs) become
+// std::runtime_error.
+inline void check(int status) {
+  if (status == VR_OK) return;
+  const std::string text = vr_strerror(status);
+  switch (status) {
+    case VR_ERR_UNALIGNED:
+    case VR_ERR_UNEVEN:
+    case VR_ERR_ALGO:
+    case VR_ERR_TOPOLOGY:
+    case VR_ERR_SUBGROUP:
+    case VR_ERR_GEOMETRY:
+      throw std::logic_error(text);
+    case VR_ERR_INVALID:
+    case VR_ERR_OVERLAP:
+      throw std::invalid_argument(text + ": " + vr_last_error_detail());
+    default:
+      throw std::runtime_error(text + ": " + vr_last_error_detail());
+  }
+}
+
+// ---- protocol tags -----------------------------------------------------------------
+// Stand-ins for the reference's wire-format classes; only their compile-time
+// constants survive (message size and wire capacity at the given sub-group size).
+template <typename T, int SubGroupSize = 16> struct Rt64 {            // rt64.hpp:334-341
+  static constexpr std::size_t messageBytes = 8;
+  static constexpr std::size_t wireCapacity = SubGroupSize * messageBytes / 2;
+  static constexpr std::size_t wireTransSize = SubGroupSize * messageBytes;
+};
+template <typename T, int SubGroupSize = 16> struct Rt64_128 {        // rt64_128.hpp:538-553
+  static constexpr std::size_t messageBytes = 128 / SubGroupSize;
+  static constexpr std::size_t wireCapacity = 120;
+  static constexpr std::size_t wireTransSize = 128;
+};
+template <typename T, int SubGroupSize = 16> struct Rt64_PCIE {       // rt64.hpp:3-20
+  static constexpr std::size_t messageBytes = 16;
+  static constexpr std::size_t wireCapacity = SubGroupSize * messageBytes / 2;
+  static constexpr std::size_t wireTransSize = SubGroupSize * messageBytes;
+};
+template <typename T, int SubGroupSize = 16> struct Rt64_128_PCIE {   // rt64_128.hpp:3-30
+  static constexpr std::size_t messageBytes = 256 / SubGroupSize;
+  static constexpr std::size_t wireCapacity = 240;
+  static constexpr std::size_t wireTransSize = 256;
+};
+
+template <typename T, int NRanks, template <typename, int> class Proto, int SubGroupSize = 16>
+struct ParallelTransmit {                                             // parallel_transmit.hpp:5-33
+  static constexpr int parallel_sg = NRanks;
+};
+template <typename T, int NRanks, template <typename, int> class Proto, int SubGroupSize = 16>
+struct SequentialTransmit {                                           // sequential_transmit.hpp:24-54
+  static constexpr int parallel_sg = 1;
+};
+template <typename T, int NRanks, template <typename, int> class Proto, int SubGroupSize = 16>
+struct RingTransmit {                                                 // sequential_transmit.hpp:226-259
+  static constexpr int parallel_sg = 1;
+};
+template <typename T, int NRanks, int SubGroupSize = 16>
+struct BisectPTransmit {                                              // bisect_transmit.hpp:3-40
+  static constexpr int BiNRanks = NRanks / 2;
+};
+
+namespace detail {
+template <template <typename, int> class A, template <typename, int> class B>
+struct same_proto { static constexpr bool value = false; };
+template <template <typename, int> class A>
+struct same_proto<A, A> { static constexpr bool value = true; };
+
+template <template <typename, int, template <typename, int> class, int> class A,
+          template <typename, int, template <typename, int> class, int> class B>
+struct same_transmit { static constexpr bool value = false; };
+template <template <typename, int, template <typename, int> class, int> class A>
+struct same_transmit<A, A> { static constexpr bool value = true; };
+
+// <Proto, Transmit> -> vr_algo, the compile-time form of allreduce.cpp:1128-1188.
+template <template <typename, int> class Proto,
+          template <typename, int, template <typename, int> class, int> class Transmit>
+constexpr int allreduce_algo() {
+  constexpr bool small = same_proto<Proto, Rt64>::value, simple = same_proto<Proto, Rt64_128>::value;
+  constexpr bool small_p = same_proto<Proto, Rt64_PCIE>::value,
+                 simple_p = same_proto<Proto, Rt64_128_PCIE>::value;
+  constexpr bool par = same_transmit<Transmit, ParallelTransmit>::value,
+                 seq = same_transmit<Transmit, SequentialTransmit>::value,
+                 ring = same_transmit<Transmit, RingTransmit>::value;
+  return par ? (small ? VR_ALGO_SMALL : simple ? VR_ALGO_SIMPLE : small_p ? VR_ALGO_SMALL_PCIE_P
+                                                                         : simple_p ? VR_ALGO_SIMPLE_PCIE_P : -1)
+       : ring ? (small_p ? VR_ALGO_SMALL_RING : simple_p ? VR_ALGO_SIMPLE_RING : -1)
+       : seq ? (small_p ? VR_ALGO_SMALL_PCIE : simple_p ? VR_ALGO_SIMPLE_PCIE : -1)
+             : -1;
+}
+}  // namespace detail
+
+// ---- the virtual ranks ------------------------------------------------------------
+// Owns the library context (scratch + flag words for the wire transport).  Stands
+// in for what main.cpp:224-283 sets up per process: scratch allocation, zeroing,
+// peer tables.
+class VirtualRanks {
+ public:
+  explicit VirtualRanks(int nranks, int device = 0) : nranks_(nranks) {
+    check(vr_ctx_create(device, nranks, &ctx_));
+  }
+  ~VirtualRanks() { vr_ctx_destroy(ctx_); }
+  VirtualRanks(const VirtualRanks &) = delete;
+  VirtualRanks &operator=(const VirtualRanks &) = delete;
+  vr_ctx *get() const { return ctx_; }
+  int size() const { return nranks_; }
+  void setTransport(int transport) { transport_ = transport; }
+  int transport() const { return transport_; }
+  void setTuning(const char *key, int value) { check(vr_ctx_set_tuning(ctx_, key, value)); }
+  // Waits for `stream` and reports a wire-transport poll time-out, if any.
+  void wait(void *stream = nullptr) { check(vr_ctx_check(ctx_, stream)); }
+
+ private:
+  vr_ctx *ctx_ = nullptr;
+  int nranks_;
+  int transport_ = VR_TRANSPORT_DEFAULT;
+};
+
+struct LaunchParam {      // the nd_range getLaunchParam returns, in sub-group units
+  std::uint32_t groups, subgroups, simd;
+};
+
+// ---- AllReduce ------------------------------------------------------------------------
+template <typename T, int NRanks, template <typename, int> class Proto,
+          template <typename, int, template <typename, int> class, int> class Transmit,
+          int SubGroupSize = 16>
+struct AllReduce {
+  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(detail::allreduce_algo<Proto, Transmit>() >= 0,
+                "this <Proto, Transmit> pair is not one the reference instantiates");
+  static_assert(SubGroupSize == 16 || SubGroupSize == 32, "Unsupported Sub-group size");
+  static constexpr int algo = detail::allreduce_algo<Proto, Transmit>();
+  static constexpr int wireCapacity = (int)Proto<T, SubGroupSize>::wireCapacity;
+
+  // Validates like the reference constructor (calcWorkSize) and remembers the
+  // buffers; throws std::logic_error with the reference's texts.
+  AllReduce(VirtualRanks &ranks, T *const inputs[], std::size_t nelems, std::uint32_t seqNo)
+      : ranks_(ranks), nelems_(nelems), seqNo_(seqNo) {
+    if (ranks.size() != NRanks) throw std::logic_error("Unsupported communication topology");
+    for (int r = 0; r < NRanks; ++r) bufs_[r] = inputs[r];
+    check(vr_check_allreduce(algo, NRanks, reinterpret_cast<const void *const *>(bufs_), nelems,
+                             &workSize_));
+  }
+
+  LaunchParam getLaunchParam(std::uint32_t &updateSeqNo) const {
+    vr_geometry g;
+    check(vr_launch_geometry(algo, NRanks, nelems_, &g));
+    updateSeqNo += g.steps;
+    return {g.groups, g.subgroups, (std::uint32_t)SubGroupSize};
+  }
+
+  // Enqueue on `stream`; in place on the constructor's buffers.
+  void operator()(void *stream = nullptr) {
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
+                       &seqNo_));
+  }
+  // "construct, then allreduce(stream, inputs, nelems)": run on other buffers of
+  // a shape this object was built for.
+  void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+                       reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
+                       &seqNo_));
+  }
+  void allreduce(void *stream, T *const inputs[], T *const outputs[], std::size_t nelems) {
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+                       reinterpret_cast<void *const *>(const_cast<T **>(inputs)),
+                       reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &seqNo_));
+  }
+
+  // The reference's "real API" (allreduce.hpp:64-74): build, size the grid,
+  // enqueue, advance `step`.
+  static void launch(VirtualRanks &ranks, T *const inputs[], std::size_t nelems,
+                     std::uint32_t &step, void *stream = nullptr) {
+    AllReduce offload(ranks, inputs, nelems, step);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+
+  std::size_t workSize() const { return workSize_; }
+  std::uint32_t seqNo() const { return seqNo_; }
+
+ private:
+  VirtualRanks &ranks_;
+  void *bufs_[VR_MAX_RANKS] = {};
+  std::size_t nelems_;
+  std::size_t workSize_ = 0;
+  std::uint32_t seqNo_;
+};
+
+// ---- bisectPAllReduce ---------------------------------------------------------------------
+template <typename T, int NRanks, template <typename, int, int> class Transmit = BisectPTransmit,
+          int SubGroupSize = 16>
+struct bisectPAllReduce {
+  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static constexpr int algo = VR_ALGO_BISECT;
+  static constexpr int BiNRanks = NRanks / 2;
+  static constexpr int wireCapacity = 120;
+
+  bisectPAllReduce(VirtualRanks &ranks, T *const inputs[], std::size_t nelems, std::uint32_t seqNo)
+      : ranks_(ranks), nelems_(nelems), seqNo_(seqNo) {
+    if (ranks.size() != NRanks) throw std::logic_error("Unsupported communication topology");
+    for (int r = 0; r < NRanks; ++r) bufs_[r] = inputs[r];
+    check(vr_check_allreduce(algo, NRanks, reinterpret_cast<const void *const *>(bufs_), nelems,
+                             &workSize_));
+  }
+  LaunchParam getLaunchParam(std::uint32_t &updateSeqNo) const {
+    vr_geometry g;
+    check(vr_launch_geometry(algo, NRanks, nelems_, &g));
+    updateSeqNo += g.steps;
+    return {g.groups, g.subgroups, (std::uint32_t)SubGroupSize};
+  }
+  void operator()(void *stream = nullptr) {
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
+                       &seqNo_));
+  }
+  void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+                       reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
+                       &seqNo_));
+  }
+  static void launch(VirtualRanks &ranks, T *const inputs[], std::size_t nelems,
+                     std::uint32_t &step, void *stream = nullptr) {
+    bisectPAllReduce offload(ranks, inputs, nelems, step);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+  std::size_t workSize() const { return workSize_; }
+
+ private:
+  VirtualRanks &ranks_;
+  void *bufs_[VR_MAX_RANKS] = {};
+  std::size_t nelems_;
+  std::size_t workSize_ = 0;
+  std::uint32_t seqNo_;
+};
+
+// ---- AllGather ----------------------------------------------------------------------------
+template <typename T, int NRanks, template <typename, int> class Proto,
+          template <typename, int, template <typename, int> class, int> class Transmit = RingTransmit,
+          int SubGroupSize = 16>
+struct AllGather {
+  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(detail::same_transmit<Transmit, RingTransmit>::value &&
+                    (detail::same_proto<Proto, Rt64_PCIE>::value ||
+                     detail::same_proto<Proto, Rt64_128_PCIE>::value),
+                "the reference gathers over RingTransmit with the *_PCIE wire formats only");
+  static constexpr int algo =
+      detail::same_proto<Proto, Rt64_PCIE>::value ? VR_ALGO_ALLGATHER_SMALL : VR_ALGO_ALLGATHER_SIMPLE;
+
+  AllGather(VirtualRanks &ranks, T *const inputs[], T *const outputs[], std::size_t nelems,
+            std::uint32_t seqNo)
+      : ranks_(ranks), nelems_(nelems), seqNo_(seqNo) {
+    if (ranks.size() != NRanks) throw std::logic_error("Unsupported communication topology");
+    for (int r = 0; r < NRanks; ++r) {
+      ins_[r] = inputs[r];
+      outs_[r] = outputs[r];
+    }
+    check(vr_check_allgather(algo, NRanks, ins_, outs_, nelems, &workSize_));
+  }
+  void operator()(void *stream = nullptr) {
+    check(vr_allgather(ranks_.get(), stream, algo, ranks_.transport(), ins_, outs_, nelems_, &seqNo_));
+  }
+  static void launch(VirtualRanks &ranks, T *const inputs[], T *const outputs[], std::size_t nelems,
+                     std::uint32_t &step, void *stream = nullptr) {
+    AllGather offload(ranks, inputs, outputs, nelems, step);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+
+ private:
+  VirtualRanks &ranks_;
+  const void *ins_[VR_MAX_RANKS] = {};
+  void *outs_[VR_MAX_RANKS] = {};
+  std::size_t nelems_;
+  std::size_t workSize_ = 0;
+  std::uint32_t seqNo_;
+};
+
+// ---- string dispatch (the test-harness flavour) --------------------------------------------
+// testTransmit<T>(algo, launchParam, ...) of allreduce.cpp:1118-1189 with a
+// user-chosen grid; unknown strings throw "Transmit type not support".
+template <typename T>
+void testTransmit(const std::string &transmitType, LaunchParam launchParam, VirtualRanks &ranks,
+                  T *const inputs[], std::size_t nelems, std::uint32_t step, void *stream = nullptr) {
+  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  int algo = -1;
+  check(vr_algo_from_string(transmitType.c_str(), &algo));
+  if (vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
+  check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transport(),
+                          reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
+                          step, launchParam.groups, launchParam.subgroups, launchParam.simd));
+}
+
+template <typename T>
+void testAllgather(const std::string &transmitType, VirtualRanks &ranks, T *const inputs[],
+                   T *const outputs[], std::size_t nelems, std::uint32_t &step,
+                   void *stream = nullptr) {
+  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  int algo = -1;
+  check(vr_algo_from_string(transmitType.c_str(), &algo));
+  if (!vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
+  check(vr_allgather(ranks.get(), stream, algo, ranks.transport(),
+                     reinterpret_cast<const void *const *>(const_cast<T **>(inputs)),
+                     reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &step));
+}
+
+}  // namespace vrank

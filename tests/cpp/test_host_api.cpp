@@ -1,0 +1,184 @@
+// Exercises the C++ host API (vrank/allreduce.hpp) the way a program written
+// against the reference's AllReduce / bisectPAllReduce / AllGather templates
+// would, and checks every result bit for bit against the CPU oracle.
+#include <stdio.h>
+#include <string.h>
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "vr_oracle.h"
+#include "vrank/allreduce.hpp"
+
+using namespace vrank;
+typedef uint16_t half_bits;   // T: any 2-byte type
+
+static int failures = 0;
+#define EXPECT(cond)                                                    \
+  do {                                                                  \
+    if (!(cond)) {                                                      \
+      printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);            \
+      ++failures;                                                       \
+    }                                                                   \
+  } while (0)
+
+struct Ranks {
+  int n;
+  size_t nelems;
+  std::vector<std::vector<half_bits>> host;
+  std::vector<half_bits *> dev;
+  Ranks(int n, size_t nelems, uint64_t seed, size_t out_mult = 1) : n(n), nelems(nelems), host(n), dev(n) {
+    for (int r = 0; r < n; ++r) {
+      host[r].resize(nelems);
+      vro_generate(host[r].data(), nelems, seed + r, VRO_DIST_NORMAL, 0.0, 1.0);
+      void *p;
+      check(vr_malloc(0, nelems * 2 * out_mult, &p));
+      dev[r] = (half_bits *)p;
+      check(vr_copy_to_device(p, host[r].data(), nelems * 2));
+    }
+  }
+  ~Ranks() { for (auto p : dev) vr_free(p); }
+  std::vector<const uint16_t *> host_ptrs() const {
+    std::vector<const uint16_t *> v;
+    for (auto &h : host) v.push_back(h.data());
+    return v;
+  }
+  size_t mismatches(const std::vector<uint16_t> &want) const {
+    size_t bad = 0;
+    std::vector<uint16_t> got(want.size());
+    for (int r = 0; r < n; ++r) {
+      check(vr_copy_to_host(got.data(), dev[r], want.size() * 2));
+      bad += vro_count_mismatch(got.data(), want.data(), want.size());
+    }
+    return bad;
+  }
+};
+
+template <typename F>
+static std::string thrown(F &&f) {
+  try { f(); } catch (const std::logic_error &e) { return e.what(); } catch (const std::exception &e) { return std::string("other: ") + e.what(); }
+  return "";
+}
+
+static int run_all() {
+  // --- AllReduce<T, 8, Rt64_128, ParallelTransmit>: construct, then call ----------------------
+  {
+    VirtualRanks ranks(8);
+    Ranks b(8, 8 * 4096 + 8 * 4 * 3, 11);
+    std::vector<uint16_t> want(b.nelems);
+    auto hp = b.host_ptrs();
+    vro_allreduce_rotated(want.data(), hp.data(), 8, b.nelems);
+    AllReduce<half_bits, 8, Rt64_128, ParallelTransmit> ar(ranks, b.dev.data(), b.nelems, 7);
+    uint32_t step = 7;
+    LaunchParam lp = ar.getLaunchParam(step);
+    EXPECT(lp.subgroups == 64 && lp.simd == 16 && step > 7);
+    ar();
+    ranks.wait();
+    EXPECT(b.mismatches(want) == 0);
+    EXPECT(ar.workSize() == b.nelems * 2 / 8);
+  }
+  // --- static launch with a running step counter (allreduce.hpp:64-74) ---------------------------
+  {
+    VirtualRanks ranks(4);
+    Ranks b(4, 4 * 1000, 21);
+    std::vector<uint16_t> want(b.nelems);
+    auto hp = b.host_ptrs();
+    vro_allreduce_rotated(want.data(), hp.data(), 4, b.nelems);
+    uint32_t step = 100;
+    AllReduce<half_bits, 4, Rt64, ParallelTransmit>::launch(ranks, b.dev.data(), b.nelems, step);
+    ranks.wait();
+    EXPECT(step > 100);
+    EXPECT(b.mismatches(want) == 0);
+  }
+  // --- ring and sequential transmits share the rotated order --------------------------------------
+  {
+    VirtualRanks ranks(8);
+    Ranks b(8, 8 * 8 * 777, 31), c(8, 8 * 8 * 777, 31);
+    std::vector<uint16_t> want(b.nelems);
+    auto hp = b.host_ptrs();
+    vro_allreduce_rotated(want.data(), hp.data(), 8, b.nelems);
+    uint32_t step = 1;
+    AllReduce<half_bits, 8, Rt64_128_PCIE, RingTransmit>::launch(ranks, b.dev.data(), b.nelems, step);
+    AllReduce<half_bits, 8, Rt64_PCIE, SequentialTransmit>::launch(ranks, c.dev.data(), c.nelems, step);
+    ranks.wait();
+    EXPECT(b.mismatches(want) == 0);
+    EXPECT(c.mismatches(want) == 0);
+  }
+  // --- bisectPAllReduce<T, 8> --------------------------------------------------------------------
+  {
+    VirtualRanks ranks(8);
+    Ranks b(8, 8 * 4 * 12345, 41);
+    std::vector<uint16_t> want(b.nelems), rot(b.nelems);
+    auto hp = b.host_ptrs();
+    vro_allreduce_bisect(want.data(), hp.data(), 8, b.nelems);
+    vro_allreduce_rotated(rot.data(), hp.data(), 8, b.nelems);
+    EXPECT(vro_count_mismatch(want.data(), rot.data(), b.nelems) > 0);
+    bisectPAllReduce<half_bits, 8> ar(ranks, b.dev.data(), b.nelems, 3);
+    ar();
+    ranks.wait();
+    EXPECT(b.mismatches(want) == 0);
+  }
+  // --- AllGather<T, 4, Rt64_128_PCIE, RingTransmit>, out of place ------------------------------------
+  {
+    VirtualRanks ranks(4);
+    Ranks in(4, 8 * 999, 51), out(4, 8 * 999, 52, 4);
+    std::vector<uint16_t> want(4 * in.nelems);
+    auto hp = in.host_ptrs();
+    vro_allgather(want.data(), hp.data(), 4, in.nelems);
+    uint32_t step = 9;
+    AllGather<half_bits, 4, Rt64_128_PCIE, RingTransmit>::launch(ranks, in.dev.data(), out.dev.data(),
+                                                                 in.nelems, step);
+    ranks.wait();
+    EXPECT(out.mismatches(want) == 0);
+  }
+  // --- string dispatch with a user grid, like main.cpp + testTransmit ---------------------------------
+  {
+    VirtualRanks ranks(8);
+    for (const char *algo : {"small", "simple", "bisect", "small_ring", "simple_pcie"}) {
+      Ranks b(8, 14336, 61);
+      std::vector<uint16_t> want(b.nelems);
+      auto hp = b.host_ptrs();
+      if (std::string(algo) == "bisect") vro_allreduce_bisect(want.data(), hp.data(), 8, b.nelems);
+      else vro_allreduce_rotated(want.data(), hp.data(), 8, b.nelems);
+      testTransmit<half_bits>(algo, {13, 8, 16}, ranks, b.dev.data(), b.nelems, 0xe00f100f);
+      ranks.wait();
+      EXPECT(b.mismatches(want) == 0);
+    }
+  }
+  // --- the reference's exceptions -------------------------------------------------------------------------
+  {
+    VirtualRanks ranks(8), two(2);
+    Ranks b(8, 8 * 64, 71);
+    EXPECT(thrown([&] { testTransmit<half_bits>("tree", {1, 4, 16}, ranks, b.dev.data(), b.nelems, 1); }) ==
+           "Transmit type not support");
+    EXPECT(thrown([&] { testTransmit<half_bits>("small", {1, 2, 16}, ranks, b.dev.data(), b.nelems, 1); }) ==
+           "Subgroup numbers must be multiple of 4");
+    EXPECT(thrown([&] { testTransmit<half_bits>("small", {1, 4, 8}, ranks, b.dev.data(), b.nelems, 1); }) ==
+           "Unsupported Sub-group size");
+    EXPECT(thrown([&] { AllReduce<half_bits, 8, Rt64, ParallelTransmit> a(ranks, b.dev.data(), 8 * 4 + 4, 1); }) ==
+           "We don't support non-even divide yet");
+    std::vector<half_bits *> odd(b.dev);
+    odd[3] = (half_bits *)((char *)odd[3] + 4);
+    EXPECT(thrown([&] { AllReduce<half_bits, 8, Rt64, ParallelTransmit> a(ranks, odd.data(), b.nelems, 1); }) ==
+           "We only support aligned pointer for now");
+    EXPECT(thrown([&] { AllReduce<half_bits, 8, Rt64, ParallelTransmit> a(two, b.dev.data(), b.nelems, 1); }) ==
+           "Unsupported communication topology");
+    EXPECT(thrown([&] { VirtualRanks three(3); }) == "Unsupported communication topology");
+  }
+  return failures;
+}
+
+int main() {
+  try {
+    if (run_all()) {
+      printf("%d check(s) failed\n", failures);
+      return 1;
+    }
+  } catch (const std::exception &e) {
+    printf("unexpected exception: %s\n", e.what());
+    return 2;
+  }
+  printf("host API ok\n");
+  return 0;
+}

@@ -1,0 +1,84 @@
+"""The C++ host API (include/vrank/allreduce.hpp) and the vr_main CLI.
+
+CPU part: both build from the committed sources and reject bad arguments with
+the reference's texts before touching a GPU.  GPU part: the C++ test program
+checks every template against the oracle, and the CLI reproduces the
+reference's -v sweep (test/test_8tile_shapes.sh) on fill_pattern inputs."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
+CPP_TEST = os.path.join(ROOT, "tests", "cpp", "test_host_api")
+
+
+def run(cmd, **kw):
+    return subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
+
+
+def test_cli_and_cpp_test_are_built():
+    assert os.path.exists(CLI), "run __graft_entry__.build()"
+    assert os.path.exists(CPP_TEST), "run make -C tests/cpp"
+
+
+def test_cli_rejects_bad_arguments_like_the_reference():
+    r = run([CLI, "-n", "1K", "-a", "tree"])
+    assert r.returncode == 1 and "Transmit type not support" in r.stdout
+    r = run([CLI, "-n", "1K", "-a", "small", "-g", "4", "-w", "2"])
+    assert r.returncode == 1 and "Subgroup numbers must be multiple of 4" in r.stdout
+    r = run([CLI, "--help"])
+    assert r.returncode == 0 and "usage" in r.stdout
+
+
+def test_header_compiles_with_plain_gxx(tmp_path):
+    src = tmp_path / "t.cpp"
+    src.write_text(
+        '#include "vrank/allreduce.hpp"\n'
+        "using namespace vrank;\n"
+        "static_assert(AllReduce<unsigned short, 8, Rt64, ParallelTransmit>::algo == VR_ALGO_SMALL, \"\");\n"
+        "static_assert(AllReduce<unsigned short, 2, Rt64_128, ParallelTransmit>::algo == VR_ALGO_SIMPLE, \"\");\n"
+        "static_assert(AllReduce<unsigned short, 8, Rt64_PCIE, RingTransmit>::algo == VR_ALGO_SMALL_RING, \"\");\n"
+        "static_assert(AllReduce<unsigned short, 8, Rt64_128_PCIE, SequentialTransmit>::algo == VR_ALGO_SIMPLE_PCIE, \"\");\n"
+        "static_assert(AllReduce<unsigned short, 2, Rt64_128, ParallelTransmit>::wireCapacity == 120, \"\");\n"
+        "static_assert(bisectPAllReduce<unsigned short, 8>::BiNRanks == 4, \"\");\n"
+        "static_assert(AllGather<unsigned short, 4, Rt64_PCIE>::algo == VR_ALGO_ALLGATHER_SMALL, \"\");\n"
+        "int main() { return 0; }\n")
+    r = run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-I", os.path.join(ROOT, "include"), str(src)])
+    assert r.returncode == 0, r.stdout
+
+
+@pytest.mark.gpu
+def test_cpp_host_api_against_oracle():
+    r = run([CPP_TEST], timeout=120)
+    assert r.returncode == 0 and "host API ok" in r.stdout, r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("world,algo", [(2, "small"), (4, "simple"), (8, "small"), (8, "simple"),
+                                        (8, "bisect"), (4, "bisect"), (8, "small_ring"),
+                                        (8, "simple_pcie"), (4, "allgather_small"),
+                                        (8, "allgather_simple")])
+def test_cli_verify_sweep(world, algo):
+    """shapes x groups x sub-groups of test/test_8tile_shapes.sh, with the
+    sub-group counts main.cpp:289-291 still accepts."""
+    shapes = [128, 256, 384, 1280, 1920, 1024, 2048, 14336, 16384]
+    msg = 8 if algo in ("small", "simple", "bisect") else 16
+    for n in shapes:
+        if not algo.startswith("allgather") and n % ((msg // 2) * world):
+            continue
+        for g, w in ((1, 4), (7, 8), (64, 64), (19, 32)):
+            r = run([CLI, "-v", "-n", str(n), "-r", str(world), "-a", algo, "-g", str(g), "-w", str(w)],
+                    timeout=60)
+            assert r.returncode == 0, r.stdout
+            assert "Error Compare" not in r.stdout and "match" in r.stdout, (n, g, w, r.stdout[-400:])
+
+
+@pytest.mark.gpu
+def test_cli_timed_run_prints_the_reference_lines():
+    r = run([CLI, "-n", "1M", "-r", "8", "-a", "bisect"], timeout=60)
+    assert r.returncode == 0, r.stdout
+    assert "---------last run------------------" in r.stdout
+    for rank in range(8):
+        assert "[%d] Running time: " % rank in r.stdout
