@@ -25,7 +25,10 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (each scaled by the same counter's reading for a plain copy of known size);
 # see profiles/.  Keyed by workload name.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/direct_allreduce_bisect_8x32MiB_hbm_traffic.md
+    "cfg3": 536923648,
+}
 
 WORKLOADS = {
     # name: (nranks, algo, nelems per rank, dist, p0, p1, seed)
@@ -179,7 +182,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["copy"],
+                    help="'copy' runs only the plain streaming copy (512 MiB per launch), the "
+                         "known-size kernel that hardware-counter readings are scaled by")
     ap.add_argument("--inplace", action="store_true",
                     help="reference semantics: results overwrite the inputs (values saturate "
                          "after a few steps; traffic is identical)")
@@ -201,6 +206,24 @@ def main():
 
     import gpu_ipc_example_amd as vr
     from gpu_ipc_example_amd import binding
+
+    if args.workload == "copy":
+        ctx = vr.VirtualRanks(8)
+        nbytes = 512 << 20
+        bufs = [binding.DeviceBuffer(nbytes) for _ in range(8)]
+        for b in bufs:
+            b.fill(0)
+        timer = binding.EventTimer(args.steps)
+        for k in range(args.steps):
+            timer.start(k)
+            ctx.stream_probe(0, bufs[(2 * k + 1) % 8].ptr, bufs[(2 * k) % 8].ptr, nbytes)
+            timer.stop(k)
+        ctx.sync()
+        ms = timer.elapsed_ms()
+        print(json.dumps({"metric": "plain_copy_bandwidth", "unit": "GB/s", "bytes_read": nbytes,
+                          "bytes_written": nbytes, "launches": args.steps,
+                          "value": round(2 * nbytes / (float(np.median(ms)) * 1e-3) / 1e9, 1)}))
+        return
 
     name = args.workload
     n, algo, ne, *_ = WORKLOADS[name]
