@@ -69,6 +69,18 @@ struct AlgoInfo {
   bool allgather;
   Order order;
   bool latency_tuned;  // "small" family: one-shot grid, cached accesses
+  WireFlow wire_flow() const {
+    if (allgather) return WIRE_ALLGATHER;
+    switch (transmit) {
+      case T_BISECT: return WIRE_BISECT;
+      case T_RING: return WIRE_RING;
+      case T_SEQUENTIAL: return WIRE_SEQUENTIAL;
+      default: return WIRE_PARALLEL;
+    }
+  }
+  // Rt64 family -> self-validating 8-byte messages; Rt64_128 family -> payload
+  // lines with release/acquire flag words.
+  WireFormat wire_format() const { return latency_tuned ? WIRE_FMT_LL : WIRE_FMT_FLAG; }
 };
 
 // message_t / wireCapacity: rt64.hpp:335-340 (8 B, 64 B), rt64_128.hpp:539-551 (8 B, 120 B),
@@ -199,13 +211,148 @@ struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
 };
 
+// Scratch of the wire transport: per virtual rank one scatter and one gather
+// sink plus their flag words (the reference's ipcbuf0 / ipcbuf1, main.cpp:241-251),
+// allocated and zeroed on first use.
+struct WireState {
+  bool ready = false;
+  void *scatter[VR_MAX_RANKS] = {}, *gather[VR_MAX_RANKS] = {};
+  void *sflag[VR_MAX_RANKS] = {}, *gflag[VR_MAX_RANKS] = {};
+  uint32_t *status = nullptr;
+  size_t sink_bytes = 0, flag_bytes = 0;
+  uint32_t block_threads = 256;   // 4 wires per work-group
+  uint32_t blocks_per_rank_max = 0;
+  bool used = false;              // a launch has written flags since the last clear
+  uint32_t next_min_seq = 0;      // smallest flag value the next launch may start at
+  int last_flow = -1, last_fmt = -1;
+};
+
 struct vr_ctx {
   int nranks = 0;
   DeviceInfo dev;
   TuningOverrides tune;
   uint32_t seq_no = 1;
   uint64_t spin_limit = 0;
+  WireState wire;
 };
+
+static const uint32_t kDefaultSpinLimit = 1u << 22;
+
+static void wire_free(vr_ctx *c) {
+  WireState &w = c->wire;
+  for (int r = 0; r < VR_MAX_RANKS; ++r) {
+    if (w.scatter[r]) (void)hipFree(w.scatter[r]);
+    if (w.gather[r]) (void)hipFree(w.gather[r]);
+    if (w.sflag[r]) (void)hipFree(w.sflag[r]);
+    if (w.gflag[r]) (void)hipFree(w.gflag[r]);
+  }
+  if (w.status) (void)hipFree(w.status);
+  w = WireState();
+}
+
+static int wire_prepare(vr_ctx *c) {
+  WireState &w = c->wire;
+  if (w.ready) return VR_OK;
+  HIP_TRY(hipSetDevice(c->dev.device));
+  const int N = c->nranks;
+  // One work-group per CU keeps every wire of every rank co-resident.
+  w.blocks_per_rank_max = (uint32_t)(c->dev.cus / N);
+  if (w.blocks_per_rank_max == 0) w.blocks_per_rank_max = 1;
+  const uint32_t wpr_max = w.blocks_per_rank_max * (w.block_threads / 64);
+  const size_t entries = (size_t)N * wpr_max + 2 * (size_t)N;
+  w.sink_bytes = entries * kWireMaxSlots * wire_slot_bytes_max();
+  w.flag_bytes = entries * kWireMaxSlots * sizeof(uint32_t);
+  for (int r = 0; r < N; ++r) {
+    HIP_TRY(hipMalloc(&w.scatter[r], w.sink_bytes));
+    HIP_TRY(hipMalloc(&w.gather[r], w.sink_bytes));
+    HIP_TRY(hipMalloc(&w.sflag[r], w.flag_bytes));
+    HIP_TRY(hipMalloc(&w.gflag[r], w.flag_bytes));
+    HIP_TRY(hipMemset(w.scatter[r], 0, w.sink_bytes));      // zeroed once, main.cpp:251
+    HIP_TRY(hipMemset(w.gather[r], 0, w.sink_bytes));
+    HIP_TRY(hipMemset(w.sflag[r], 0, w.flag_bytes));
+    HIP_TRY(hipMemset(w.gflag[r], 0, w.flag_bytes));
+  }
+  HIP_TRY(hipMalloc((void **)&w.status, 256));
+  HIP_TRY(hipMemset(w.status, 0, 256));
+  HIP_TRY(hipDeviceSynchronize());
+  w.ready = true;
+  return VR_OK;
+}
+
+// Forget every flag ever written (asynchronous, ordered on `s`).
+static int wire_clear(vr_ctx *c, hipStream_t s) {
+  WireState &w = c->wire;
+  for (int r = 0; r < c->nranks; ++r) {
+    hipError_t e = launch_wire_clear(s, w.scatter[r], w.sink_bytes);
+    if (e == hipSuccess) e = launch_wire_clear(s, w.gather[r], w.sink_bytes);
+    if (e == hipSuccess) e = launch_wire_clear(s, w.sflag[r], w.flag_bytes);
+    if (e == hipSuccess) e = launch_wire_clear(s, w.gflag[r], w.flag_bytes);
+    if (e != hipSuccess) return fail_hip(e, "launch_wire_clear");
+  }
+  w.used = false;
+  return VR_OK;
+}
+
+// Launches one wire-transport collective.  `user_wires` (0 = automatic) is the
+// number of sub-groups per rank a caller asked for with -g/-w.  Returns through
+// *flags_used how many consecutive flag values the launch consumes.
+static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
+                       const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t seq,
+                       uint32_t user_wires, uint32_t *flags_used) {
+  if (seq == 0)
+    return fail(VR_ERR_INVALID, "sequence number 0 cannot be told from freshly zeroed scratch");
+  if (int rc = wire_prepare(c)) return rc;
+  WireState &w = c->wire;
+  const int N = c->nranks;
+  const WireFlow flow = a->wire_flow();
+  const WireFormat fmt = a->wire_format();
+  const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
+  const uint32_t waves_per_block = w.block_threads / 64;
+  const uint32_t wpr_limit = w.blocks_per_rank_max * waves_per_block / psg * psg;
+  if (wpr_limit < psg) return fail(VR_ERR_INVALID, "device too small for this rank count");
+  const uint32_t wire_bytes = wire_bytes_per_step(fmt, vec_halves);
+  const size_t wires_per_chunk = div_up(chunk_bytes, wire_bytes);
+  if (wires_per_chunk == 0) { *flags_used = 0; return VR_OK; }
+  size_t want = user_wires ? (size_t)user_wires / psg * psg : wires_per_chunk * psg;
+  if (want < psg) want = psg;
+  if (want > wpr_limit) want = wpr_limit;
+  const uint32_t wpr = (uint32_t)want;
+  const uint32_t blocks_per_rank = (uint32_t)div_up(wpr, waves_per_block);
+  const size_t steps = div_up(wires_per_chunk, wpr / psg);
+  const uint32_t nslot_min = 4;
+  *flags_used = (uint32_t)((steps - 1) / nslot_min + 1);
+
+  // Flags must strictly increase on every slot; a different flow or format
+  // re-interprets the sinks, so start those from a clean slate too.
+  const bool moved_back = w.used && (int32_t)(seq - w.next_min_seq) < 0;
+  if (moved_back || (w.used && (w.last_flow != (int)flow || w.last_fmt != (int)fmt)))
+    if (int rc = wire_clear(c, s)) return rc;
+
+  WireArgs args;
+  memset(&args, 0, sizeof args);
+  args.in = in;
+  args.out = out;
+  for (int r = 0; r < N; ++r) {
+    args.scatter.p[r] = w.scatter[r];
+    args.gather.p[r] = w.gather[r];
+    args.sflag.p[r] = w.sflag[r];
+    args.gflag.p[r] = w.gflag[r];
+  }
+  args.chunk_bytes = chunk_bytes;
+  args.waves_per_rank = wpr;
+  args.seq = seq;
+  const uint64_t limit = c->spin_limit ? c->spin_limit : kDefaultSpinLimit;
+  args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
+  args.status = w.status;
+  hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args);
+  if (e != hipSuccess) return fail_hip(e, "launch_wire (cooperative)");
+  w.used = true;
+  w.next_min_seq = seq + *flags_used;
+  w.last_flow = (int)flow;
+  w.last_fmt = (int)fmt;
+  return VR_OK;
+}
+
 
 extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   if (!out) return fail(VR_ERR_INVALID, "null out");
@@ -234,6 +381,7 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
 
 extern "C" int vr_ctx_destroy(vr_ctx *ctx) {
   if (!ctx) return VR_OK;
+  wire_free(ctx);
   delete ctx;
   return VR_OK;
 }
@@ -386,11 +534,18 @@ static int resolve_transport(const AlgoInfo *a, int transport, int *out) {
   return VR_OK;
 }
 
+// Runs one all-reduce; *advance receives how far the sequence number moves.
 static int run_allreduce(vr_ctx *ctx, hipStream_t s, const Prepared &p, int transport,
-                         const Tuning &t, uint32_t seq_no) {
-  (void)seq_no;
-  if (transport == VR_TRANSPORT_WIRE)
-    return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
+                         const Tuning &t, uint32_t seq_no, uint32_t user_wires, uint32_t *advance) {
+  *advance = p.geom.steps;          // getLaunchParam: updateSeqNo += nSteps
+  if (transport == VR_TRANSPORT_WIRE) {
+    uint32_t used = 0;
+    if (int rc = wire_launch(ctx, s, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, seq_no,
+                             user_wires, &used))
+      return rc;
+    if (used > *advance) *advance = used;
+    return VR_OK;
+  }
   hipError_t e = launch_direct_allreduce(s, ctx->dev, t, ctx->nranks, p.a->order, p.in, p.out,
                                          p.chunk_elems, p.vec_halves);
   if (e != hipSuccess) return fail_hip(e, "launch_direct_allreduce");
@@ -405,8 +560,12 @@ extern "C" int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, 
   if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
   const uint32_t start = *seq;
-  if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr, tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place), start)) return rc;
-  *seq = start + p.geom.steps;   // getLaunchParam: updateSeqNo += nSteps
+  uint32_t advance = 0;
+  if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr,
+                             tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place),
+                             start, 0, &advance))
+    return rc;
+  *seq = start + advance;
   return VR_OK;
 }
 
@@ -433,7 +592,11 @@ extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transp
   t.unroll = 1;
   t.oneshot = 0;
   t.force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
-  return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no);
+  // Wire transport: groups x subgroups is the number of sub-groups (wires) per rank.
+  const uint64_t wires = (uint64_t)groups * subgroups;
+  uint32_t advance = 0;
+  return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no,
+                       wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &advance);
 }
 
 struct PreparedGather {
@@ -483,14 +646,21 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
                             uint32_t *seq_no) {
   PreparedGather p;
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
-  if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
+  uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
+  if (transport == VR_TRANSPORT_WIRE) {
+    uint32_t used = 0;
+    if (int rc = wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves, *seq,
+                             0, &used))
+      return rc;
+    *seq += used > p.geom.steps ? used : p.geom.steps;
+    return VR_OK;
+  }
   if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
   const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
   hipError_t e = launch_direct_allgather((hipStream_t)stream, ctx->dev,
                                          tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false),
                                          ctx->nranks, p.in, p.out, nelems, p.vec_halves);
   if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
-  uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
   *seq += p.geom.steps;
   return VR_OK;
 }
@@ -498,7 +668,17 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
 extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
   if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  return VR_OK;
+  WireState &w = ctx->wire;
+  if (!w.ready) return VR_OK;
+  uint32_t status = 0;
+  HIP_TRY(hipMemcpy(&status, w.status, sizeof status, hipMemcpyDeviceToHost));
+  if (status == 0) return VR_OK;
+  // A poll gave up: results of that launch are undefined and half-delivered
+  // messages may still sit in the sinks.  Start over from clean scratch.
+  HIP_TRY(hipMemset(w.status, 0, 256));
+  if (int rc = wire_clear(ctx, (hipStream_t)stream)) return rc;
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return fail(VR_ERR_TIMEOUT, "a wire-transport poll exceeded the spin limit; scratch was reset");
 }
 
 // ---------------------------------------------------------------------------------
@@ -544,8 +724,9 @@ extern "C" int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transp
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
     const uint32_t start = ctx->seq_no;
-    int rc = run_allreduce(ctx, s, p, tr, t, start);
-    ctx->seq_no = start + p.geom.steps;
+    uint32_t advance = 0;
+    int rc = run_allreduce(ctx, s, p, tr, t, start, 0, &advance);
+    ctx->seq_no = start + advance;
     return rc;
   });
 }
@@ -555,11 +736,16 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
                                  int iters, float *ms_out) {
   PreparedGather p;
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
-  if (transport == VR_TRANSPORT_WIRE) return fail(VR_ERR_INVALID, "wire transport is not built into this library yet");
   const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
   const Tuning t = tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false);
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
+    if (transport == VR_TRANSPORT_WIRE) {
+      uint32_t used = 0;
+      int rc = wire_launch(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, ctx->seq_no, 0, &used);
+      ctx->seq_no += used > p.geom.steps ? used : p.geom.steps;
+      return rc;
+    }
     hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);
     return e == hipSuccess ? VR_OK : fail_hip(e, "launch_direct_allgather");
   });

@@ -50,4 +50,31 @@ hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const T
 hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, void *dst,
                        const void *src, size_t bytes, int mode = 0);
 
+
+// Wire transport ------------------------------------------------------------------
+enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER };
+enum WireFormat : int {
+  WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
+  WIRE_FMT_FLAG = 1,  // 16 B payload lines + one release/acquire flag word per message (Rt64_128 family)
+};
+constexpr int kWireUnroll = 2;       // messages per lane and step
+constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
+
+struct WireArgs {
+  PtrTable in, out;          // per-rank input / output
+  PtrTable scatter, gather;  // per-rank sinks
+  PtrTable sflag, gflag;     // per-rank flag words (WIRE_FMT_FLAG)
+  size_t chunk_bytes;        // bytes per rank-chunk (all-gather: bytes of one slice)
+  uint32_t waves_per_rank;   // wires each virtual rank runs (multiple of the flow's waves per column)
+  uint32_t seq;              // first flag value of this launch
+  uint32_t spin_limit;
+  uint32_t *status;          // non-zero once any poll gave up
+};
+
+uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves);
+uint32_t wire_slot_bytes_max();
+hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
+                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args);
+hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
+
 }  // namespace vr

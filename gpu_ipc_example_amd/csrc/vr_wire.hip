@@ -1,0 +1,482 @@
+// Wire transport: the reference's message-passing stage structure on one GPU.
+//
+// One persistent, cooperatively launched kernel holds the work-groups of ALL
+// virtual ranks (block b belongs to rank b % N).  A wavefront plays the part of
+// a reference sub-group ("wire"): it loads its rank's input, pushes messages
+// into peers' scatter/gather sinks in device scratch, polls its own sinks, adds
+// in the reference's order and stores.  Sink indexing, slot rotation and flag
+// values follow parallel_transmit.hpp:47-58,75,93-122, sequential_transmit.hpp:
+// 57-81,112-206 (Sequential), 262-278,333-516 (Ring) and bisect_transmit.hpp:
+// 286-424,432-481, re-tiled for 64-lane wavefronts.
+//
+// Two wire formats:
+//   WireLL    (Rt64 family, rt64.hpp:334-341): every 8-byte store carries 4 bytes
+//             of payload and the 4-byte flag, so a message validates itself; the
+//             receiver re-polls until a wave-wide vote says every lane's flag is
+//             the expected one (the sub-group vote of parallel_transmit.hpp:95-101).
+//             Needs nothing but 8-byte store atomicity.
+//   WireFlag  (Rt64_128 family): full 16-byte-per-lane payload lines plus ONE flag
+//             word per message in a separate array.  The sender stores the
+//             payload, executes an agent-scope release fence, then lane 0 stores
+//             the flag; the receiver polls the flag word with agent-scope loads
+//             and executes an acquire fence before reading the payload.  This
+//             replaces the reference's two embedded flags per 128 bytes
+//             (rt64_128.hpp:544-553), whose correctness rests on 64-byte store
+//             atomicity that gfx950 does not promise.
+//
+// Every poll is bounded: after `spin_limit` unsuccessful polls (or as soon as
+// another wave has given up) a wave records a time-out in the status word and
+// runs to completion without waiting again, so the grid always drains.
+
+#include "vr_internal.h"
+
+namespace vr {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+
+#define VR_AGENT __HIP_MEMORY_SCOPE_AGENT
+
+struct Spin {
+  uint32_t limit;
+  uint32_t *status;
+  uint32_t lane;
+  bool dead;
+  // Called after an unsuccessful poll (wave-uniform).  True = stop waiting.
+  __device__ __forceinline__ bool give_up(uint32_t &polls) {
+    ++polls;
+    if (polls >= limit ||
+        ((polls & 63u) == 0 && __hip_atomic_load(status, __ATOMIC_RELAXED, VR_AGENT) != 0)) {
+      dead = true;
+      if (lane == 0) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, VR_AGENT);
+      return true;
+    }
+    __builtin_amdgcn_s_sleep(1);
+    return false;
+  }
+};
+
+// ---- wire formats ---------------------------------------------------------------
+
+template <int U>
+struct WireLL {
+  static constexpr uint32_t kWireBytes = 64u * 4u * U;   // payload one wave moves per step
+  static constexpr uint32_t kSlotBytes = 64u * 8u * U;   // message bytes in the sink
+  struct Reg {
+    uint32_t d[U];
+  };
+
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+    Reg r;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * 4u;
+      r.d[u] = off < left ? *reinterpret_cast<const uint32_t *>(p + off) : 0u;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * 4u;
+      if (off < left) *reinterpret_cast<uint32_t *>(p + off) = r.d[u];
+    }
+  }
+  // v = m + v, element-wise binary16, message on the left (rt64.hpp:452-463).
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const h2 s = __builtin_bit_cast(h2, m.d[u]) + __builtin_bit_cast(h2, v.d[u]);
+      v.d[u] = __builtin_bit_cast(uint32_t, s);
+    }
+  }
+  static __device__ __forceinline__ void send(char *slot, uint32_t *, const Reg &v, uint32_t flag,
+                                              uint32_t lane) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint64_t msg = (uint64_t)v.d[u] | ((uint64_t)flag << 32);
+      __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, msg, __ATOMIC_RELAXED,
+                         VR_AGENT);
+    }
+  }
+  static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
+                                              uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint64_t msg = __hip_atomic_load(reinterpret_cast<const uint64_t *>(slot) + u * 64 + lane,
+                                               __ATOMIC_RELAXED, VR_AGENT);
+        v.d[u] = (uint32_t)msg;
+        ok = ok && (uint32_t)(msg >> 32) == flag;
+      }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
+};
+
+template <int U, typename V>
+struct WireFlag {
+  static constexpr uint32_t kWireBytes = 64u * (uint32_t)sizeof(V) * U;
+  static constexpr uint32_t kSlotBytes = kWireBytes;
+  struct Reg {
+    V d[U];
+  };
+
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+    Reg r;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
+      V z = {};
+      r.d[u] = off < left ? *reinterpret_cast<const V *>(p + off) : z;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
+      if (off < left) *reinterpret_cast<V *>(p + off) = r.d[u];
+    }
+  }
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:947-957
+#pragma unroll
+    for (int u = 0; u < U; ++u) v.d[u] = m.d[u] + v.d[u];
+  }
+  static __device__ __forceinline__ void send(char *slot, uint32_t *flagword, const Reg &v,
+                                              uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) reinterpret_cast<V *>(slot)[u * 64 + lane] = v.d[u];
+    // Every lane's payload store must be visible device-wide before the flag is.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    if (lane == 0) __hip_atomic_store(flagword, flag, __ATOMIC_RELAXED, VR_AGENT);
+  }
+  static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *flagword, Reg &v,
+                                              uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    // All lanes read the same word, so the loop condition is wave-uniform.
+    while (__hip_atomic_load(flagword, __ATOMIC_RELAXED, VR_AGENT) != flag) {
+      if (spin.give_up(polls)) return false;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+    for (int u = 0; u < U; ++u) v.d[u] = reinterpret_cast<const V *>(slot)[u * 64 + lane];
+    return true;
+  }
+};
+
+// ---- sinks --------------------------------------------------------------------------
+
+template <typename W, int NSLOT>
+struct Sinks {
+  const WireArgs &a;
+  __device__ __forceinline__ char *scat(int rank, uint32_t entry, uint32_t s) const {
+    return static_cast<char *>(a.scatter.p[rank]) + ((size_t)entry * NSLOT + s) * W::kSlotBytes;
+  }
+  __device__ __forceinline__ char *gath(int rank, uint32_t entry, uint32_t s) const {
+    return static_cast<char *>(a.gather.p[rank]) + ((size_t)entry * NSLOT + s) * W::kSlotBytes;
+  }
+  __device__ __forceinline__ uint32_t *sflag(int rank, uint32_t entry, uint32_t s) const {
+    return static_cast<uint32_t *>(a.sflag.p[rank]) + (size_t)entry * NSLOT + s;
+  }
+  __device__ __forceinline__ uint32_t *gflag(int rank, uint32_t entry, uint32_t s) const {
+    return static_cast<uint32_t *>(a.gflag.p[rank]) + (size_t)entry * NSLOT + s;
+  }
+};
+
+#define VR_WAVE_PROLOGUE                                                             \
+  const int r = blockIdx.x % N;                                                      \
+  const uint32_t lane = threadIdx.x & 63u;                                           \
+  const uint32_t wid = (blockIdx.x / N) * (blockDim.x >> 6) + (threadIdx.x >> 6);    \
+  if (wid >= a.waves_per_rank) return;                                               \
+  Spin spin{a.spin_limit, a.status, lane, false};                                    \
+  const size_t chunk = a.chunk_bytes
+
+static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, uint32_t wire) {
+  const size_t left = chunk - off;
+  return left < wire ? (uint32_t)left : wire;
+}
+
+// ---- ParallelTransmit::run (parallel_transmit.hpp:63-131) -----------------------------
+// N waves per wire column; wave y serves chunk y.  The wave with y == rank owns
+// the column's reduction for its rank's chunk.
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
+  constexpr int NSLOT = 8;
+  VR_WAVE_PROLOGUE;
+  const Sinks<W, NSLOT> sk{a};
+  const uint32_t y = wid % N, x_id = wid / N * N;
+  const size_t columns = a.waves_per_rank / N;
+  const char *src = static_cast<const char *>(a.in.p[r]) + y * chunk;
+  char *dst = static_cast<char *>(a.out.p[r]) + y * chunk;
+  uint32_t t = 0;
+  for (size_t off = (size_t)(wid / N) * W::kWireBytes; off < chunk; off += columns * W::kWireBytes, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    typename W::Reg v = W::load(src + off, left, lane);
+    if ((int)y != r) {                               // scatter, then wait for the gather
+      W::send(sk.scat(y, x_id + r, s), sk.sflag(y, x_id + r, s), v, flag, lane);
+      W::recv(sk.gath(r, x_id + y, s), sk.gflag(r, x_id + y, s), v, flag, lane, spin);
+    } else {                                         // wait, reduce, broadcast
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        typename W::Reg m;
+        W::recv(sk.scat(r, x_id + next, s), sk.sflag(r, x_id + next, s), m, flag, lane, spin);
+        W::add(v, m);
+      }
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        W::send(sk.gath(next, x_id + r, s), sk.gflag(next, x_id + r, s), v, flag, lane);
+      }
+    }
+    W::store(dst + off, left, lane, v);
+  }
+}
+
+// ---- SequentialTransmit::run (sequential_transmit.hpp:83-207) -----------------------------
+// One wave does everything its rank owes a wire column, peer after peer.
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
+  constexpr int NSLOT = 4;
+  VR_WAVE_PROLOGUE;
+  const Sinks<W, NSLOT> sk{a};
+  const uint32_t wpr = a.waves_per_rank;
+  const char *src = static_cast<const char *>(a.in.p[r]);
+  char *dst = static_cast<char *>(a.out.p[r]);
+  uint32_t t = 0;
+  for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      const typename W::Reg p = W::load(src + next * chunk + off, left, lane);
+      W::send(sk.scat(next, r * wpr + wid, s), sk.sflag(next, r * wpr + wid, s), p, flag, lane);
+    }
+    typename W::Reg v = W::load(src + r * chunk + off, left, lane);
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      typename W::Reg m;
+      W::recv(sk.scat(r, next * wpr + wid, s), sk.sflag(r, next * wpr + wid, s), m, flag, lane, spin);
+      W::add(v, m);
+    }
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      W::send(sk.gath(next, r * wpr + wid, s), sk.gflag(next, r * wpr + wid, s), v, flag, lane);
+    }
+    W::store(dst + r * chunk + off, left, lane, v);
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      typename W::Reg m;
+      W::recv(sk.gath(r, next * wpr + wid, s), sk.gflag(r, next * wpr + wid, s), m, flag, lane, spin);
+      W::store(dst + next * chunk + off, left, lane, m);
+    }
+  }
+}
+
+// ---- RingTransmit::runAllreduce (sequential_transmit.hpp:429-472) ----------------------------
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
+  constexpr int NSLOT = 4;
+  VR_WAVE_PROLOGUE;
+  const Sinks<W, NSLOT> sk{a};
+  const uint32_t wpr = a.waves_per_rank;
+  const int next = (r + 1) % N;
+  const char *src = static_cast<const char *>(a.in.p[r]);
+  char *dst = static_cast<char *>(a.out.p[r]);
+  uint32_t t = 0;
+  for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = (a.seq + t) % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    int peer = r;
+    typename W::Reg v = W::load(src + peer * chunk + off, left, lane);           // step 0: send
+    W::send(sk.scat(next, peer * wpr + wid, s), sk.sflag(next, peer * wpr + wid, s), v, flag, lane);
+    for (int i = 1; i < N - 1; ++i) {                                            // reduce and forward
+      peer = (r + N - i) % N;
+      v = W::load(src + peer * chunk + off, left, lane);
+      typename W::Reg m;
+      W::recv(sk.scat(r, peer * wpr + wid, s), sk.sflag(r, peer * wpr + wid, s), m, flag, lane, spin);
+      W::add(v, m);
+      W::send(sk.scat(next, peer * wpr + wid, s), sk.sflag(next, peer * wpr + wid, s), v, flag, lane);
+    }
+    peer = (r + 1) % N;                                                          // last add, start the gather ring
+    v = W::load(src + peer * chunk + off, left, lane);
+    {
+      typename W::Reg m;
+      W::recv(sk.scat(r, peer * wpr + wid, s), sk.sflag(r, peer * wpr + wid, s), m, flag, lane, spin);
+      W::add(v, m);
+    }
+    W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
+    W::store(dst + peer * chunk + off, left, lane, v);
+    for (int i = 1; i < N - 1; ++i) {                                            // forward and write back
+      peer = (r + 1 + N - i) % N;
+      W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
+      W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
+      W::store(dst + peer * chunk + off, left, lane, v);
+    }
+    peer = (r + 2) % N;                                                          // last hop: write back only
+    W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
+    W::store(dst + peer * chunk + off, left, lane, v);
+  }
+}
+
+// ---- RingTransmit::runAllgather (sequential_transmit.hpp:474-516) ----------------------------
+// chunk = bytes of one rank's slice; out[r] holds N slices.
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
+  constexpr int NSLOT = 4;
+  VR_WAVE_PROLOGUE;
+  const Sinks<W, NSLOT> sk{a};
+  const uint32_t wpr = a.waves_per_rank;
+  const int next = (r + 1) % N;
+  const char *src = static_cast<const char *>(a.in.p[r]);
+  char *dst = static_cast<char *>(a.out.p[r]);
+  uint32_t t = 0;
+  for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = (a.seq + t) % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    int peer = r;
+    typename W::Reg v = W::load(src + off, left, lane);
+    if (src != dst + (size_t)peer * chunk) W::store(dst + (size_t)peer * chunk + off, left, lane, v);
+    W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
+    for (int i = 1; i < N - 1; ++i) {
+      peer = (r + N - i) % N;
+      W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
+      W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
+      W::store(dst + (size_t)peer * chunk + off, left, lane, v);
+    }
+    peer = (r + 1) % N;
+    W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
+    W::store(dst + (size_t)peer * chunk + off, left, lane, v);
+  }
+}
+
+// ---- bisectPAllReduce::operator() (allreduce.hpp:275-296, bisect_transmit.hpp:286-424) -------------
+// N/2 waves per wire column; even ranks own the first half of the buffer, odd
+// ranks the second; pair exchange first, then the flat exchange among the ranks
+// of the same parity.
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
+  constexpr int NSLOT = 8, B = N / 2;
+  VR_WAVE_PROLOGUE;
+  const Sinks<W, NSLOT> sk{a};
+  const uint32_t y = wid % B, wg = wid / B * B;
+  const size_t columns = a.waves_per_rank / B;
+  const uint32_t far_base = a.waves_per_rank + B;     // the far sinks sit behind the close ones
+  const int h = r & 1, l = r >> 1, pair = r ^ 1;
+  const size_t close_off = (h ? (size_t)B * chunk : 0) + y * chunk;
+  const size_t far_off = (h ? 0 : (size_t)B * chunk) + y * chunk;
+  const char *src = static_cast<const char *>(a.in.p[r]);
+  char *dst = static_cast<char *>(a.out.p[r]);
+  uint32_t t = 0;
+  for (size_t off = (size_t)(wid / B) * W::kWireBytes; off < chunk; off += columns * W::kWireBytes, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    {                                                 // scatterFar
+      const typename W::Reg f = W::load(src + far_off + off, left, lane);
+      W::send(sk.scat(pair, far_base + wid, s), sk.sflag(pair, far_base + wid, s), f, flag, lane);
+    }
+    typename W::Reg v = W::load(src + close_off + off, left, lane);
+    {                                                 // pair sum
+      typename W::Reg m;
+      W::recv(sk.scat(r, far_base + wid, s), sk.sflag(r, far_base + wid, s), m, flag, lane, spin);
+      W::add(v, m);
+    }
+    if ((int)y != l) {
+      const int owner = 2 * (int)y + h;
+      W::send(sk.scat(owner, wg + l, s), sk.sflag(owner, wg + l, s), v, flag, lane);
+      W::recv(sk.gath(r, wg + y, s), sk.gflag(r, wg + y, s), v, flag, lane, spin);
+    } else {
+      for (int i = 0; i < B - 1; ++i) {
+        const int l_next = (l + i + 1) % B;
+        typename W::Reg m;
+        W::recv(sk.scat(r, wg + l_next, s), sk.sflag(r, wg + l_next, s), m, flag, lane, spin);
+        W::add(v, m);
+      }
+      for (int i = 0; i < B - 1; ++i) {
+        const int nx = (r + i * 2 + 2) % N;
+        W::send(sk.gath(nx, wg + l, s), sk.gflag(nx, wg + l, s), v, flag, lane);
+      }
+    }
+    W::send(sk.gath(pair, far_base + wid, s), sk.gflag(pair, far_base + wid, s), v, flag, lane);
+    W::store(dst + close_off + off, left, lane, v);
+    {                                                 // pollFarGatherOutput
+      typename W::Reg m;
+      W::recv(sk.gath(r, far_base + wid, s), sk.gflag(r, far_base + wid, s), m, flag, lane, spin);
+      W::store(dst + far_off + off, left, lane, m);
+    }
+  }
+}
+
+// Clears the sinks' flag state on the stream (a fill kernel rather than a memset
+// node, so that callers may capture the launch sequence in a graph).
+__global__ void k_wire_clear(uint64_t *p, size_t n64) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n64;
+       i += (size_t)gridDim.x * blockDim.x)
+    p[i] = 0;
+}
+
+// ---- host side --------------------------------------------------------------------------
+
+template <typename W>
+static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 grid, dim3 block,
+                              WireArgs &args) {
+  void *kargs[] = {&args};
+  const void *fn = nullptr;
+#define VR_PICK(NN)                                                                         \
+  case NN:                                                                                  \
+    switch (flow) {                                                                         \
+      case WIRE_PARALLEL: fn = reinterpret_cast<const void *>(&k_wire_parallel<NN, W>); break;   \
+      case WIRE_SEQUENTIAL: fn = reinterpret_cast<const void *>(&k_wire_sequential<NN, W>); break; \
+      case WIRE_RING: fn = reinterpret_cast<const void *>(&k_wire_ring<NN, W>); break;           \
+      case WIRE_ALLGATHER: fn = reinterpret_cast<const void *>(&k_wire_allgather<NN, W>); break;  \
+      case WIRE_BISECT:                                                                     \
+        if constexpr (NN >= 4) fn = reinterpret_cast<const void *>(&k_wire_bisect<NN, W>);  \
+        break;                                                                              \
+    }                                                                                       \
+    break;
+  switch (nranks) {
+    VR_PICK(2)
+    VR_PICK(4)
+    VR_PICK(8)
+    VR_PICK(16)
+    default: break;
+  }
+#undef VR_PICK
+  if (!fn) return hipErrorInvalidValue;
+  // Cooperative launch: the runtime refuses a grid that cannot be co-resident,
+  // which is what makes spinning on another work-group's progress safe.
+  return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+}
+
+uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
+  switch (fmt) {
+    case WIRE_FMT_LL: return WireLL<kWireUnroll>::kWireBytes;
+    default:
+      return vec_halves == 8 ? WireFlag<kWireUnroll, h8>::kWireBytes
+                             : WireFlag<kWireUnroll, h4>::kWireBytes;
+  }
+}
+
+uint32_t wire_slot_bytes_max() { return WireFlag<kWireUnroll, h8>::kSlotBytes; }
+
+hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
+                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args) {
+  const dim3 grid(blocks_per_rank * nranks), block(block_threads);
+  if (fmt == WIRE_FMT_LL) return launch_flow<WireLL<kWireUnroll>>(s, flow, nranks, grid, block, args);
+  if (vec_halves == 8) return launch_flow<WireFlag<kWireUnroll, h8>>(s, flow, nranks, grid, block, args);
+  return launch_flow<WireFlag<kWireUnroll, h4>>(s, flow, nranks, grid, block, args);
+}
+
+hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {
+  if (bytes == 0) return hipSuccess;
+  hipLaunchKernelGGL(k_wire_clear, dim3(1024), dim3(256), 0, s, static_cast<uint64_t *>(p), bytes / 8);
+  return hipGetLastError();
+}
+
+}  // namespace vr

@@ -1,0 +1,203 @@
+"""GPU parity tests of the wire transport (message passing through scratch with
+flags, one persistent kernel holding every virtual rank's work-groups).  Same
+oracle, same bit-exact bar as the direct transport."""
+import numpy as np
+import pytest
+
+import gpu_ipc_example_amd as vr
+from tests import vr_helpers as H
+from tests.oracle_lib import DIST_NORMAL, DIST_UNIFORM
+
+pytestmark = pytest.mark.gpu
+WIRE = vr.TRANSPORT_WIRE
+
+
+@pytest.fixture(scope="module")
+def ctxs():
+    made = {n: vr.VirtualRanks(n) for n in (2, 4, 8, 16)}
+    yield made
+    for c in made.values():
+        c.close()
+
+
+def h(x):
+    return int(np.array([x], np.float16).view(np.uint16)[0])
+
+
+def per_chunk(out, nranks):
+    chunk = len(out) // nranks
+    return [float(out[c * chunk:(c + 1) * chunk].view(np.float16)[0]) for c in range(nranks)]
+
+
+@pytest.mark.parametrize("algo", ["small", "simple", "parallel", "bisect", "small_ring", "simple_ring",
+                                  "small_pcie", "simple_pcie"])
+def test_kat_n8(ctxs, algo):
+    ins = [np.full(1024, h(v), np.uint16) for v in (2048, 0, 1, 0, 1, 0, 0, 0)]
+    got, _ = H.run_allreduce(ctxs[8], algo, ins, transport=WIRE)
+    want = ([2048, 2050, 2048, 2048, 2048, 2050, 2048, 2048] if algo == "bisect"
+            else [2048, 2050, 2050, 2048, 2048, 2048, 2048, 2048])
+    for g in got:
+        assert per_chunk(g, 8) == want
+        assert (g.reshape(8, -1) == g.reshape(8, -1)[:, :1]).all()
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("algo", H.ROTATED_ALGOS + ("parallel", "bisect"))
+def test_random_all_algos(ctxs, oracle, nranks, algo):
+    if algo == "bisect" and nranks < 4:
+        pytest.skip("bisect needs >= 4 ranks")
+    msg = 16 if ("pcie" in algo or "ring" in algo) else 8
+    unit = (msg // 2) * nranks
+    for k, n in enumerate((unit, unit * 3, unit * 129, unit * 1000 + unit, 1 << 20)):
+        n = (n // unit) * unit
+        ins = H.make_inputs(oracle, nranks, n, 3000 * nranks + 10 * k)
+        want = H.expected(oracle, algo, ins)
+        got, _ = H.run_allreduce(ctxs[nranks], algo, ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, want, "%s N=%d n=%d in-place" % (algo, nranks, n))
+        got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=False, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, want, "%s N=%d n=%d out-of-place" % (algo, nranks, n))
+        for a, b in zip(kept, ins):
+            assert (a == b).all()
+
+
+def test_bisect_16_ranks(ctxs, oracle):
+    for n in (64, 64 * 77, 1 << 18):
+        ins = H.make_inputs(oracle, 16, n, 78)
+        got, _ = H.run_allreduce(ctxs[16], "bisect", ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, oracle.bisect(ins))
+
+
+@pytest.mark.parametrize("algo", ["simple", "bisect", "small"])
+def test_eight_byte_granularity(ctxs, oracle, algo):
+    for n in (32 * 1, 32 * 3, 32 * 1001):
+        ins = H.make_inputs(oracle, 8, n, 41 + n)
+        got, _ = H.run_allreduce(ctxs[8], algo, ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "n=%d" % n)
+    ins = H.make_inputs(oracle, 8, 1 << 16, 9)
+    got, _ = H.run_allreduce(ctxs[8], algo, ins, offset_bytes=8, transport=WIRE)
+    H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "offset 8")
+
+
+@pytest.mark.parametrize("groups", [1, 2, 4, 8, 16, 32, 64, 7, 13, 15, 17, 19])
+def test_result_independent_of_grid(ctxs, oracle, groups):
+    n = 14336
+    ins = H.make_inputs(oracle, 8, n, 501)
+    for algo in ("small", "simple", "bisect", "simple_ring"):
+        want = H.expected(oracle, algo, ins)
+        for subgroups in (4, 8, 32, 64):
+            got, _ = H.run_allreduce(ctxs[8], algo, ins, grid=(groups, subgroups, 16), transport=WIRE)
+            H.assert_all_ranks_equal(oracle, got, want, "%s g=%d w=%d" % (algo, groups, subgroups))
+
+
+def test_many_launches_reuse_slots_and_flags(ctxs, oracle):
+    """Back-to-back launches without host synchronisation: slot rings wrap, the
+    sequence number keeps the flags apart."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    ctx = ctxs[8]
+    n = 8 * 4096 * 6            # several steps per launch at the automatic grid
+    for algo in ("small", "simple", "bisect", "small_ring", "simple_pcie"):
+        base = H.make_inputs(oracle, 8, n, 900)
+        cur = [a.copy() for a in base]
+        bufs = [DeviceBuffer(n * 2) for _ in range(8)]
+        for b, a in zip(bufs, cur):
+            b.upload(a)
+        rounds = 5
+        for _ in range(rounds):
+            ctx.allreduce(algo, [b.ptr for b in bufs], n, transport=WIRE)     # in place, async
+        ctx.check()
+        for _ in range(rounds):
+            s = H.expected(oracle, algo, cur)
+            cur = [s.copy() for _ in range(8)]
+        for b in bufs:
+            assert oracle.count_mismatch(b.download(np.uint16, n), cur[0]) == 0, algo
+            b.free()
+
+
+def test_sequence_number_moving_backwards_is_safe(ctxs, oracle):
+    ctx = ctxs[8]
+    ins = H.make_inputs(oracle, 8, 8 * 4096, 77)
+    want = oracle.rotated(ins)
+    for seq in (0xE00F100F, 0xE00F100F, 5, 5, 1):          # repeats and regressions
+        got, _ = H.run_allreduce(ctx, "simple", ins, grid=(16, 8, 16), transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, want)
+        src = H.RankBuffers(8, len(ins[0]))
+        src.upload(ins)
+        ctx.allreduce_grid("simple", src.ptrs, len(ins[0]), 16, 8, 16, transport=WIRE, seq_no=seq)
+        ctx.check()
+        H.assert_all_ranks_equal(oracle, src.download(), want, "seq %#x" % seq)
+        src.free()
+    with pytest.raises(vr.VRError) as e:
+        src = H.RankBuffers(8, len(ins[0]))
+        ctx.allreduce_grid("simple", src.ptrs, len(ins[0]), 16, 8, 16, transport=WIRE, seq_no=0)
+    assert e.value.code == "INVALID"
+
+
+def test_poll_timeout_is_reported_and_recoverable(ctxs, oracle):
+    """A spin limit of one poll makes some wave give up before its message has
+    arrived; every wave still runs to completion, the context reports the
+    time-out, and the next launch works."""
+    ctx = vr.VirtualRanks(8)
+    ins = H.make_inputs(oracle, 8, 1 << 20, 31)
+    ctx.set_spin_limit(1)
+    timed_out = False
+    for algo in ("simple_ring", "small_ring", "bisect"):
+        try:
+            H.run_allreduce(ctx, algo, ins, transport=WIRE)
+        except vr.VRError as e:
+            assert e.code == "TIMEOUT"
+            timed_out = True
+    assert timed_out
+    ctx.set_spin_limit(0)
+    got, _ = H.run_allreduce(ctx, "simple_ring", ins, transport=WIRE)
+    H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins))
+    ctx.close()
+
+
+def test_config3_bisect_32mib_wire(ctxs, oracle):
+    ins = H.make_inputs(oracle, 8, 16777216, 3000, DIST_NORMAL, 0.0, 0.02)
+    got, _ = H.run_allreduce(ctxs[8], "bisect", ins, transport=WIRE)
+    H.assert_all_ranks_equal(oracle, got, oracle.bisect(ins))
+
+
+def test_parallel_defaults_to_wire_and_sweep_sizes(ctxs, oracle):
+    for p in range(11, 24, 2):
+        n = 1 << p
+        ins = H.make_inputs(oracle, 8, n, 5100 + p)
+        got, _ = H.run_allreduce(ctxs[8], "parallel", ins)          # default transport
+        H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins), "n=%d" % n)
+
+
+def run_allgather_wire(ctx, algo, ins, alias_own_slot=False):
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    N, n = ctx.nranks, len(ins[0])
+    outs = [DeviceBuffer(N * n * 2 + 64) for _ in range(N)]
+    for o in outs:
+        o.fill(0x01)
+    if alias_own_slot:
+        in_ptrs = [outs[r].ptr + r * n * 2 for r in range(N)]
+        for r in range(N):
+            outs[r].upload(ins[r], r * n * 2)
+        srcs = []
+    else:
+        srcs = [DeviceBuffer(n * 2 + 64) for _ in range(N)]
+        for s, a in zip(srcs, ins):
+            s.upload(a)
+        in_ptrs = [s.ptr for s in srcs]
+    ctx.allgather(algo, in_ptrs, [o.ptr for o in outs], n, transport=WIRE)
+    ctx.check()
+    got = [o.download(np.uint16, N * n) for o in outs]
+    for b in outs + srcs:
+        b.free()
+    return got
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_allgather_wire(ctxs, oracle, nranks, algo):
+    for n in (8, 8 * 15, 8 * 1237, 1 << 16, 1 << 20):
+        ins = H.make_inputs(oracle, nranks, n, 71 + n, DIST_UNIFORM, -2.0, 2.0)
+        want = oracle.allgather(ins)
+        for alias in (False, True):
+            got = run_allgather_wire(ctxs[nranks], algo, ins, alias)
+            for r in range(nranks):
+                assert (got[r] == want).all(), (n, r, alias)
