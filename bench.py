@@ -177,6 +177,53 @@ def cpu_baseline(name, budget_s):
     }
 
 
+def sweep(vr, binding, args):
+    """BASELINE config 5: 8 virtual ranks, per-rank sizes 4 KiB ... 256 MiB in powers of
+    two, in place on one buffer set, N(0,1) inputs.  One line of JSON: GB/s and us per
+    size for each protocol, and the sizes at which the fastest protocol changes."""
+    n = 8
+    ctx = vr.VirtualRanks(n)
+    max_bytes = 256 << 20
+    host = binding.generate(max_bytes // 2, 5000, 1, 0.0, 1.0)
+    bufs = [binding.DeviceBuffer(max_bytes) for _ in range(n)]
+    protos = [("small", vr.TRANSPORT_DIRECT), ("simple", vr.TRANSPORT_DIRECT),
+              ("bisect", vr.TRANSPORT_DIRECT), ("parallel", vr.TRANSPORT_WIRE)]
+    if args.sweep_wire:
+        protos += [(a, vr.TRANSPORT_WIRE) for a in ("small", "simple", "bisect", "small_ring",
+                                                     "simple_ring", "small_pcie", "simple_pcie")]
+    curves = {}
+    sizes = [1 << p for p in range(12, 29)]
+    for algo, tr in protos:
+        key = algo + ("@wire" if tr == vr.TRANSPORT_WIRE and algo != "parallel" else "")
+        rows = []
+        for S in sizes:
+            ne = S // 2
+            for b in bufs:
+                b.upload(host[:ne])
+            ptrs = [b.ptr for b in bufs]
+            direct = tr == vr.TRANSPORT_DIRECT
+            iters = (200 if S <= (1 << 22) else 40) if direct else (30 if S <= (1 << 22) else 5)
+            ctx.time_allreduce(algo, ptrs, ne, 3, transport=tr)
+            ms = ctx.time_allreduce(algo, ptrs, ne, iters, transport=tr)
+            ctx.check()
+            us = float(np.median(ms)) * 1e3
+            rows.append({"bytes_per_rank": S, "us": round(us, 2),
+                         "GBps": round(2 * n * S / (us * 1e-6) / 1e9, 1)})
+        curves[key] = rows
+    best = []
+    for i, S in enumerate(sizes):
+        name = min(curves, key=lambda k: curves[k][i]["us"])
+        best.append(name)
+    crossovers = [{"bytes_per_rank": sizes[i], "from": best[i - 1], "to": best[i]}
+                  for i in range(1, len(sizes)) if best[i] != best[i - 1]]
+    print(json.dumps({"metric": "allreduce_GBps_vs_size_8vrank_fp16", "unit": "GB/s",
+                      "note": "in place on one buffer set: sizes up to 16 MiB/rank are served by "
+                              "the caches, 64 MiB/rank and above stream from HBM; times are HIP-event "
+                              "times of single launches (~2 us of event overhead included)",
+                      "curves": curves, "fastest": dict(zip(map(str, sizes), best)),
+                      "crossovers": crossovers}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -198,6 +245,11 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--latency-iters", type=int, default=1000)
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VAL")
+    ap.add_argument("--sweep", action="store_true",
+                    help="GB/s-vs-size curves of small / simple / bisect / parallel and their "
+                         "crossover sizes instead of the headline measurement")
+    ap.add_argument("--sweep-wire", action="store_true",
+                    help="with --sweep: add every message-passing flow to the curves")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every virtual rank lives in one MI355X's HBM; "
@@ -206,6 +258,10 @@ def main():
 
     import gpu_ipc_example_amd as vr
     from gpu_ipc_example_amd import binding
+
+    if args.sweep:
+        sweep(vr, binding, args)
+        return
 
     if args.workload == "copy":
         ctx = vr.VirtualRanks(8)

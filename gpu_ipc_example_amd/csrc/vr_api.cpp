@@ -78,9 +78,9 @@ struct AlgoInfo {
       default: return WIRE_PARALLEL;
     }
   }
-  // Rt64 family -> self-validating 8-byte messages; Rt64_128 family -> payload
-  // lines with release/acquire flag words.
-  WireFormat wire_format() const { return latency_tuned ? WIRE_FMT_LL : WIRE_FMT_FLAG; }
+  // Rt64 family -> self-validating 8-byte messages; Rt64_128 family -> 64-byte
+  // segments of 15 payload dwords and a flag.
+  WireFormat wire_format() const { return latency_tuned ? WIRE_FMT_LL : WIRE_FMT_LL64; }
 };
 
 // message_t / wireCapacity: rt64.hpp:335-340 (8 B, 64 B), rt64_128.hpp:539-551 (8 B, 120 B),
@@ -209,6 +209,7 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 // User overrides of the launch heuristics; -1 = let the library decide.
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
+  int wire_fenced = -1, wire_cooperative = -1;
 };
 
 // Scratch of the wire transport: per virtual rank one scatter and one gather
@@ -305,7 +306,8 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   WireState &w = c->wire;
   const int N = c->nranks;
   const WireFlow flow = a->wire_flow();
-  const WireFormat fmt = a->wire_format();
+  WireFormat fmt = a->wire_format();
+  if (fmt == WIRE_FMT_LL64 && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
   const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
   const uint32_t waves_per_block = w.block_threads / 64;
   const uint32_t wpr_limit = w.blocks_per_rank_max * waves_per_block / psg * psg;
@@ -344,8 +346,10 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const uint64_t limit = c->spin_limit ? c->spin_limit : kDefaultSpinLimit;
   args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
   args.status = w.status;
-  hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args);
-  if (e != hipSuccess) return fail_hip(e, "launch_wire (cooperative)");
+  const bool cooperative = c->tune.wire_cooperative != 0;
+  hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args,
+                             cooperative);
+  if (e != hipSuccess) return fail_hip(e, cooperative ? "launch_wire (cooperative)" : "launch_wire");
   w.used = true;
   w.next_min_seq = seq + *flags_used;
   w.last_flow = (int)flow;
@@ -402,6 +406,8 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "nt_load")) return &ctx->tune.nt_load;
   if (!strcmp(key, "nt_store")) return &ctx->tune.nt_store;
   if (!strcmp(key, "oneshot")) return &ctx->tune.oneshot;
+  if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
+  if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   return nullptr;
 }
 
@@ -415,7 +421,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
     if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
       return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
-    if ((!strcmp(key, "nt_load") || !strcmp(key, "nt_store") || !strcmp(key, "oneshot")) &&
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "nt_store") || !strcmp(key, "oneshot") ||
+         !strcmp(key, "wire_fenced") || !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
   }

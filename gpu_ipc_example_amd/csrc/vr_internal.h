@@ -55,9 +55,9 @@ hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, vo
 enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER };
 enum WireFormat : int {
   WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
-  WIRE_FMT_FLAG = 1,  // 16 B payload lines + one release/acquire flag word per message (Rt64_128 family)
+  WIRE_FMT_LL64 = 1,  // 60 B payload + 4 B flag per 64-byte segment (Rt64_128 family)
+  WIRE_FMT_FLAG = 2,  // 16 B payload lines + one fenced flag word per message
 };
-constexpr int kWireUnroll = 2;       // messages per lane and step
 constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
 
 struct WireArgs {
@@ -73,8 +73,10 @@ struct WireArgs {
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves);
 uint32_t wire_slot_bytes_max();
+// cooperative: hipLaunchCooperativeKernel instead of a plain launch.
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args);
+                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
+                       bool cooperative);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
 
 }  // namespace vr

@@ -9,20 +9,16 @@
 // 57-81,112-206 (Sequential), 262-278,333-516 (Ring) and bisect_transmit.hpp:
 // 286-424,432-481, re-tiled for 64-lane wavefronts.
 //
-// Two wire formats:
+// Three wire formats:
 //   WireLL    (Rt64 family, rt64.hpp:334-341): every 8-byte store carries 4 bytes
 //             of payload and the 4-byte flag, so a message validates itself; the
 //             receiver re-polls until a wave-wide vote says every lane's flag is
 //             the expected one (the sub-group vote of parallel_transmit.hpp:95-101).
 //             Needs nothing but 8-byte store atomicity.
-//   WireFlag  (Rt64_128 family): full 16-byte-per-lane payload lines plus ONE flag
-//             word per message in a separate array.  The sender stores the
-//             payload, executes an agent-scope release fence, then lane 0 stores
-//             the flag; the receiver polls the flag word with agent-scope loads
-//             and executes an acquire fence before reading the payload.  This
-//             replaces the reference's two embedded flags per 128 bytes
-//             (rt64_128.hpp:544-553), whose correctness rests on 64-byte store
-//             atomicity that gfx950 does not promise.
+//   WireLL64  (Rt64_128 family): 15 payload dwords + 1 flag per 64-byte segment.
+//   WireFlag  (assumption-free alternative for the Rt64_128 family): payload lines
+//             plus a separate flag word, ordered by agent-scope release/acquire
+//             fences.
 //
 // Every poll is bounded: after `spin_limit` unsuccessful polls (or as soon as
 // another wave has given up) a wave records a time-out in the status word and
@@ -119,6 +115,95 @@ struct WireLL {
   }
 };
 
+// Rt64_128 re-tiled for wavefronts (rt64_128.hpp:538-553, 635-685, 724-802): the
+// reference packs 30 payload dwords and a flag at dword 15 and at dword 31 into a
+// 128-byte message, one flag per 64-byte half "because a 128-byte transaction is
+// not atomic across HBM channels".  Here a wave's message is 512 bytes = eight
+// 64-byte segments; the eight lanes of a segment store 8 bytes each in ONE store
+// instruction, lanes 0..6 two payload dwords, lane 7 one payload dword and the
+// flag: 15 payload dwords + 1 flag per 64 bytes, the reference's 93.75 %.  A
+// receiver's lane trusts its segment once the segment's flag lane has seen the
+// expected flag (wave vote).  Like the reference's format this rests on a
+// 64-byte segment written by one instruction becoming visible as a whole.
+template <int U>
+struct WireLL64 {
+  static constexpr uint32_t kWireBytes = 480u * U;
+  static constexpr uint32_t kSlotBytes = 512u * U;
+  struct Reg {
+    uint32_t d[U][2];
+  };
+  // Index of the lane's first payload dword inside message u.
+  static __device__ __forceinline__ uint32_t dword0(int u, uint32_t lane) {
+    return (uint32_t)u * 120u + (lane >> 3) * 15u + (lane & 7u) * 2u;
+  }
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+    Reg r;
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
+    const bool two = (lane & 7u) != 7u;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = dword0(u, lane);
+      r.d[u][0] = 4u * i < left ? q[i] : 0u;
+      r.d[u][1] = (two && 4u * (i + 1) < left) ? q[i + 1] : 0u;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+    uint32_t *q = reinterpret_cast<uint32_t *>(p);
+    const bool two = (lane & 7u) != 7u;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = dword0(u, lane);
+      if (4u * i < left) q[i] = r.d[u][0];
+      if (two && 4u * (i + 1) < left) q[i + 1] = r.d[u][1];
+    }
+  }
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:947-957
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {   // the flag lane's second dword is rewritten by send()
+        const h2 s = __builtin_bit_cast(h2, m.d[u][k]) + __builtin_bit_cast(h2, v.d[u][k]);
+        v.d[u][k] = __builtin_bit_cast(uint32_t, s);
+      }
+  }
+  static __device__ __forceinline__ void send(char *slot, uint32_t *, const Reg &v, uint32_t flag,
+                                              uint32_t lane) {
+    const bool flag_lane = (lane & 7u) == 7u;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint64_t msg = (uint64_t)v.d[u][0] | ((uint64_t)(flag_lane ? flag : v.d[u][1]) << 32);
+      __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, msg, __ATOMIC_RELAXED,
+                         VR_AGENT);
+    }
+  }
+  static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
+                                              uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    const bool flag_lane = (lane & 7u) == 7u;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint64_t msg = __hip_atomic_load(reinterpret_cast<const uint64_t *>(slot) + u * 64 + lane,
+                                               __ATOMIC_RELAXED, VR_AGENT);
+        v.d[u][0] = (uint32_t)msg;
+        v.d[u][1] = (uint32_t)(msg >> 32);
+        ok = ok && (!flag_lane || v.d[u][1] == flag);
+      }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
+};
+
+// Flag-word format: full 16-byte-per-lane payload lines plus ONE flag word per
+// message in a separate array, ordered by agent-scope fences: the sender stores
+// the payload, executes a release fence (L2 write-back), then lane 0 stores the
+// flag; the receiver polls the flag word and executes an acquire fence (cache
+// invalidate) before it loads the payload.  Assumes nothing about store
+// atomicity, and pays two cache-maintenance operations per message for it.
 template <int U, typename V>
 struct WireFlag {
   static constexpr uint32_t kWireBytes = 64u * (uint32_t)sizeof(V) * U;
@@ -144,7 +229,7 @@ struct WireFlag {
       if (off < left) *reinterpret_cast<V *>(p + off) = r.d[u];
     }
   }
-  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:947-957
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
 #pragma unroll
     for (int u = 0; u < U; ++u) v.d[u] = m.d[u] + v.d[u];
   }
@@ -152,7 +237,6 @@ struct WireFlag {
                                               uint32_t flag, uint32_t lane) {
 #pragma unroll
     for (int u = 0; u < U; ++u) reinterpret_cast<V *>(slot)[u * 64 + lane] = v.d[u];
-    // Every lane's payload store must be visible device-wide before the flag is.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     if (lane == 0) __hip_atomic_store(flagword, flag, __ATOMIC_RELAXED, VR_AGENT);
   }
@@ -421,11 +505,16 @@ __global__ void k_wire_clear(uint64_t *p, size_t n64) {
     p[i] = 0;
 }
 
+// Messages per lane and step for each format; every slot stays within 2 KiB.
+constexpr int kUnrollLL = 4;     // 1 KiB payload in a 2 KiB message
+constexpr int kUnrollLL64 = 4;   // 1920 B payload in a 2 KiB message
+constexpr int kUnrollFlag = 2;   // 2 KiB payload (16-byte lanes), flag word elsewhere
+
 // ---- host side --------------------------------------------------------------------------
 
 template <typename W>
 static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 grid, dim3 block,
-                              WireArgs &args) {
+                              WireArgs &args, bool cooperative) {
   void *kargs[] = {&args};
   const void *fn = nullptr;
 #define VR_PICK(NN)                                                                         \
@@ -450,27 +539,36 @@ static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 gri
 #undef VR_PICK
   if (!fn) return hipErrorInvalidValue;
   // Cooperative launch: the runtime refuses a grid that cannot be co-resident,
-  // which is what makes spinning on another work-group's progress safe.
-  return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+  // which is what makes spinning on another work-group's progress safe.  The
+  // plain launch is for callers that accept "at most one work-group per CU on
+  // an otherwise idle device" as that guarantee and want the shorter launch path.
+  if (cooperative) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+  return hipLaunchKernel(fn, grid, block, kargs, 0, s);
 }
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   switch (fmt) {
-    case WIRE_FMT_LL: return WireLL<kWireUnroll>::kWireBytes;
+    case WIRE_FMT_LL: return WireLL<kUnrollLL>::kWireBytes;
+    case WIRE_FMT_LL64: return WireLL64<kUnrollLL64>::kWireBytes;
     default:
-      return vec_halves == 8 ? WireFlag<kWireUnroll, h8>::kWireBytes
-                             : WireFlag<kWireUnroll, h4>::kWireBytes;
+      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8>::kWireBytes
+                             : WireFlag<kUnrollFlag, h4>::kWireBytes;
   }
 }
 
-uint32_t wire_slot_bytes_max() { return WireFlag<kWireUnroll, h8>::kSlotBytes; }
+uint32_t wire_slot_bytes_max() { return WireFlag<kUnrollFlag, h8>::kSlotBytes; }
 
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args) {
+                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
+                       bool cooperative) {
   const dim3 grid(blocks_per_rank * nranks), block(block_threads);
-  if (fmt == WIRE_FMT_LL) return launch_flow<WireLL<kWireUnroll>>(s, flow, nranks, grid, block, args);
-  if (vec_halves == 8) return launch_flow<WireFlag<kWireUnroll, h8>>(s, flow, nranks, grid, block, args);
-  return launch_flow<WireFlag<kWireUnroll, h4>>(s, flow, nranks, grid, block, args);
+  if (fmt == WIRE_FMT_LL)
+    return launch_flow<WireLL<kUnrollLL>>(s, flow, nranks, grid, block, args, cooperative);
+  if (fmt == WIRE_FMT_LL64)
+    return launch_flow<WireLL64<kUnrollLL64>>(s, flow, nranks, grid, block, args, cooperative);
+  if (vec_halves == 8)
+    return launch_flow<WireFlag<kUnrollFlag, h8>>(s, flow, nranks, grid, block, args, cooperative);
+  return launch_flow<WireFlag<kUnrollFlag, h4>>(s, flow, nranks, grid, block, args, cooperative);
 }
 
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {

@@ -156,7 +156,12 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
 /* Tuning knobs for the direct kernels (benchmark sweeps).  Unknown keys are
  * VR_ERR_INVALID.  Keys: "block" (threads per work-group), "waves_per_cu"
  * (persistent grid size = CUs * this / waves per block), "unroll" (16-byte
- * vectors in flight per lane and rank), "nt_load", "nt_store" (0/1). */
+ * vectors in flight per lane and rank), "nt_load", "nt_store", "oneshot" (0/1);
+ * for the wire transport "wire_fenced" (1 = the Rt64_128 family sends payload
+ * lines with a separate flag word ordered by agent-scope release/acquire fences
+ * instead of 64-byte segments with an embedded flag) and
+ * "wire_cooperative" (0 = plain launch instead of a cooperative one).
+ * -1 restores the library's own choice. */
 int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value);
 int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);
 

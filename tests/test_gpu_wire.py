@@ -201,3 +201,52 @@ def test_allgather_wire(ctxs, oracle, nranks, algo):
             got = run_allgather_wire(ctxs[nranks], algo, ins, alias)
             for r in range(nranks):
                 assert (got[r] == want).all(), (n, r, alias)
+
+
+@pytest.mark.parametrize("algo", ["simple", "parallel", "bisect", "simple_ring", "simple_pcie",
+                                  "simple_pcie_p"])
+def test_fenced_flag_word_format(oracle, algo):
+    """The Rt64_128 family can also travel as payload lines + a separate flag word
+    ordered by agent-scope release/acquire fences (no store-atomicity assumption)."""
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_fenced=1)
+    for n in (64, 64 * 129, 1 << 18, 32 * 1001):
+        if algo in ("simple_ring", "simple_pcie", "simple_pcie_p") and n % 64:
+            continue
+        ins = H.make_inputs(oracle, 8, n, 6000 + n)
+        got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+    ctx.close()
+
+
+def test_plain_launch_instead_of_cooperative(oracle):
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_cooperative=0)
+    for algo in ("small", "simple", "bisect", "small_ring"):
+        ins = H.make_inputs(oracle, 8, 1 << 18, 6100)
+        got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), algo)
+    ctx.close()
+
+
+@pytest.mark.parametrize("algo", ["simple", "bisect", "simple_ring", "small"])
+def test_embedded_flag_formats_under_repetition(ctxs, oracle, algo):
+    """Many launches over the same sinks: every 64-byte segment (Rt64_128 family)
+    and every 8-byte message (Rt64 family) must arrive whole every time."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    ctx = ctxs[8]
+    n = 8 * 8192
+    ins = H.make_inputs(oracle, 8, n, 6200)
+    want = H.expected(oracle, algo, ins)
+    src = [DeviceBuffer(n * 2) for _ in range(8)]
+    dst = [DeviceBuffer(n * 2) for _ in range(8)]
+    for b, a in zip(src, ins):
+        b.upload(a)
+    for it in range(150):
+        ctx.allreduce(algo, [b.ptr for b in src], n, outs=[b.ptr for b in dst], transport=WIRE)
+        if it % 10 == 9:
+            ctx.check()
+            for r, b in enumerate(dst):
+                assert oracle.count_mismatch(b.download(np.uint16, n), want) == 0, (algo, it, r)
+    for b in src + dst:
+        b.free()
