@@ -455,7 +455,10 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   const size_t kMall = 256ull << 20;
   Tuning t;
   t.block = 256;
-  t.waves_per_cu = 8;
+  // The all-reduce keeps N loads per lane in flight and is DRAM-efficiency bound
+  // from 8 waves per CU on; the all-gather has one load per lane and needs the
+  // CU's full 32 waves to cover the latency.
+  t.waves_per_cu = a->allgather ? 32 : 8;
   t.unroll = 1;
   if (a->latency_tuned) {
     // "small" family: every lane makes one trip; results stay cacheable for the
