@@ -251,9 +251,21 @@ static void wire_free(vr_ctx *c) {
   w = WireState();
 }
 
+static int wire_allocate(vr_ctx *c);
+
 static int wire_prepare(vr_ctx *c) {
+  if (c->wire.ready) return VR_OK;
+  const int rc = wire_allocate(c);
+  if (rc != VR_OK) {          // do not keep a half-built scratch set around
+    const std::string detail = g_detail;
+    wire_free(c);
+    g_detail = detail;
+  }
+  return rc;
+}
+
+static int wire_allocate(vr_ctx *c) {
   WireState &w = c->wire;
-  if (w.ready) return VR_OK;
   HIP_TRY(hipSetDevice(c->dev.device));
   const int N = c->nranks;
   // One work-group per CU keeps every wire of every rank co-resident.
@@ -441,6 +453,14 @@ extern "C" int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value) {
 // hot path
 // ---------------------------------------------------------------------------------
 
+// Every launch path starts here: kernels go to the context's device whatever the
+// calling thread's current device is.
+static int use_device(const vr_ctx *ctx) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  HIP_TRY(hipSetDevice(ctx->dev.device));
+  return VR_OK;
+}
+
 static bool ranges_partially_overlap(const void *a, const void *b, size_t bytes) {
   if (a == b) return false;
   const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
@@ -502,7 +522,7 @@ struct Prepared {
 
 static int prepare_allreduce(vr_ctx *ctx, int algo, void *const bufs[], void *const outs[],
                              size_t nelems, Prepared *p) {
-  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (int rc = use_device(ctx)) return rc;
   const AlgoInfo *a = algo_info(algo);
   if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
   const int N = ctx->nranks;
@@ -618,7 +638,7 @@ struct PreparedGather {
 
 static int prepare_allgather(vr_ctx *ctx, int algo, const void *const inputs[],
                              void *const outputs[], size_t nelems, PreparedGather *p) {
-  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (int rc = use_device(ctx)) return rc;
   const AlgoInfo *a = algo_info(algo);
   if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
   const int N = ctx->nranks;
@@ -676,7 +696,7 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
 }
 
 extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
-  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (int rc = use_device(ctx)) return rc;
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
   WireState &w = ctx->wire;
   if (!w.ready) return VR_OK;
@@ -765,6 +785,7 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
 // 16-byte vectors per lane in flight (what measured best for a plain copy).
 static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, Tuning *t) {
   if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
+  if (int rc = use_device(ctx)) return rc;
   if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16)
     return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
   Tuning d;

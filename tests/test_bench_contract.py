@@ -1,0 +1,24 @@
+"""bench.py contract checks that need no GPU."""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_algorithmic_bytes_match_the_metric_definition():
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.algorithmic_bytes("cfg3") == 2 * 8 * 32 * 2**20          # 2*N*S
+    assert bench.algorithmic_bytes("cfg2") == 2 * 8 * 2**20
+    assert bench.algorithmic_bytes("cfg4") == 4 * 8 * 2**20 + 4 * 4 * 8 * 2**20   # N*S + N*N*S
+    assert bench.WORKLOADS["cfg3"][:3] == (8, "bisect", 16777216)
+    assert bench.WORKLOADS["cfg2"][:3] == (8, "small", 524288)
+    assert bench.WORKLOADS["cfg4"][:3] == (4, "allgather_simple", 4194304)
