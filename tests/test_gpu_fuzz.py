@@ -1,0 +1,47 @@
+"""Randomised parity sweep: random world size, protocol, transport, element
+count, alignment and in/out-of-place choice, each checked bit for bit against
+the oracle.  Seeds are fixed, so a failure names a reproducible case."""
+import random
+
+import numpy as np
+import pytest
+
+import gpu_ipc_example_amd as vr
+from tests import vr_helpers as H
+
+pytestmark = pytest.mark.gpu
+
+ALGOS8 = ("small", "simple", "bisect", "parallel")
+ALGOS16 = ("small_pcie_p", "simple_pcie_p", "small_ring", "simple_ring", "small_pcie", "simple_pcie")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_cases(oracle, seed):
+    rng = random.Random(1000 + seed)
+    ctxs = {n: vr.VirtualRanks(n) for n in (2, 4, 8, 16)}
+    for case in range(40):
+        algo = rng.choice(ALGOS8 + ALGOS16)
+        nranks = rng.choice((4, 8, 16) if algo == "bisect" else (2, 4, 8))
+        msg_halves = 4 if algo in ALGOS8 else 8
+        unit = msg_halves * nranks
+        n = unit * rng.choice((1, 2, 3, 5, 17, 63, 64, 65, 257, 1000, 4099, 16384 // unit + 1,
+                               rng.randrange(1, 40000)))
+        transport = rng.choice((vr.TRANSPORT_DIRECT, vr.TRANSPORT_WIRE))
+        inplace = rng.random() < 0.5
+        offset = rng.choice((0, 0, 0, 16, 8 if msg_halves == 4 else 16, 32))
+        grid = None
+        if rng.random() < 0.4:
+            grid = (rng.choice((1, 2, 3, 7, 16, 33, 64)), rng.choice((4, 8, 12, 32, 64)), rng.choice((16, 32)))
+        ins = H.make_inputs(oracle, nranks, n, 10_000 * seed + 37 * case,
+                            p1=rng.choice((0.02, 1.0, 30.0, 3000.0)))
+        what = "seed=%d case=%d %s N=%d n=%d transport=%d inplace=%s offset=%d grid=%s" % (
+            seed, case, algo, nranks, n, transport, inplace, offset, grid)
+        print(what, flush=True)
+        got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=inplace, transport=transport,
+                                    offset_bytes=offset, grid=grid)
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), what)
+        if kept is not None:
+            for a, b in zip(kept, ins):
+                assert (a == b).all(), what
+    for c in ctxs.values():
+        c.close()
