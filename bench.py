@@ -178,7 +178,7 @@ def cpu_baseline(name, budget_s):
 
 
 def sweep(vr, binding, args):
-    """BASELINE config 5: 8 virtual ranks, per-rank sizes 4 KiB ... 256 MiB in powers of
+    """The size sweep: 8 virtual ranks, per-rank sizes 4 KiB ... 256 MiB in powers of
     two, in place on one buffer set, N(0,1) inputs.  One line of JSON: GB/s and us per
     size for each protocol, and the sizes at which the fastest protocol changes."""
     n = 8

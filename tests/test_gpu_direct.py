@@ -200,7 +200,7 @@ def test_special_values(ctxs, oracle):
         H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), algo)
 
 
-# ---- BASELINE configurations at full size ------------------------------------------------------
+# ---- the five benchmark configurations at full size ------------------------------------------------------
 
 def test_config1_two_ranks_simple(ctxs, oracle):
     ins = H.make_inputs(oracle, 2, 16384, 1234, DIST_UNIFORM, -1.0, 1.0)
