@@ -67,6 +67,10 @@ def lib():
         "vr_ctx_create": (i, [i, i, vpp]),
         "vr_ctx_destroy": (i, [vp]),
         "vr_ctx_nranks": (i, [vp]),
+        "vr_ctx_set_dtype": (i, [vp, i]),
+        "vr_ctx_get_dtype": (i, [vp]),
+        "vr_fill_pattern_dt": (None, [i, C.POINTER(C.c_uint16), i, sz]),
+        "vr_generate_dt": (None, [i, C.POINTER(C.c_uint16), sz, C.c_uint64, i, C.c_double, C.c_double]),
         "vr_algo_from_string": (i, [C.c_char_p, C.POINTER(i)]),
         "vr_algo_name": (C.c_char_p, [i]),
         "vr_algo_is_allgather": (i, [i]),
@@ -148,15 +152,18 @@ def launch_geometry(algo, nranks, nelems):
     return g.groups, g.subgroups, g.steps
 
 
-def fill_pattern(rank, n):
+DTYPE_F16, DTYPE_BF16 = 0, 1
+
+
+def fill_pattern(rank, n, dtype=DTYPE_F16):
     a = np.empty(n, np.uint16)
-    lib().vr_fill_pattern(a.ctypes.data_as(C.POINTER(C.c_uint16)), rank, n)
+    lib().vr_fill_pattern_dt(dtype, a.ctypes.data_as(C.POINTER(C.c_uint16)), rank, n)
     return a
 
 
-def generate(n, seed, dist, p0, p1):
+def generate(n, seed, dist, p0, p1, dtype=DTYPE_F16):
     a = np.empty(n, np.uint16)
-    lib().vr_generate(a.ctypes.data_as(C.POINTER(C.c_uint16)), n, seed, dist, p0, p1)
+    lib().vr_generate_dt(dtype, a.ctypes.data_as(C.POINTER(C.c_uint16)), n, seed, dist, p0, p1)
     return a
 
 
@@ -229,6 +236,9 @@ class VirtualRanks:
             self.close()
         except Exception:
             pass
+
+    def set_dtype(self, dtype):
+        _check(lib().vr_ctx_set_dtype(self._h, dtype))
 
     def set_tuning(self, **kw):
         for k, v in kw.items():

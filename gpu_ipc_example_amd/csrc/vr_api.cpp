@@ -234,6 +234,7 @@ struct vr_ctx {
   TuningOverrides tune;
   uint32_t seq_no = 1;
   uint64_t spin_limit = 0;
+  DType dtype = DT_F16;
   WireState wire;
 };
 
@@ -360,7 +361,7 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   args.status = w.status;
   const bool cooperative = c->tune.wire_cooperative != 0;
   hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args,
-                             cooperative);
+                             cooperative, c->dtype);
   if (e != hipSuccess) return fail_hip(e, cooperative ? "launch_wire (cooperative)" : "launch_wire");
   w.used = true;
   w.next_min_seq = seq + *flags_used;
@@ -403,6 +404,15 @@ extern "C" int vr_ctx_destroy(vr_ctx *ctx) {
 }
 
 extern "C" int vr_ctx_nranks(const vr_ctx *ctx) { return ctx ? ctx->nranks : 0; }
+
+extern "C" int vr_ctx_set_dtype(vr_ctx *ctx, int dtype) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (dtype != VR_DTYPE_F16 && dtype != VR_DTYPE_BF16) return fail(VR_ERR_INVALID, "unknown element type");
+  ctx->dtype = dtype == VR_DTYPE_BF16 ? DT_BF16 : DT_F16;
+  return VR_OK;
+}
+
+extern "C" int vr_ctx_get_dtype(const vr_ctx *ctx) { return ctx ? (int)ctx->dtype : -1; }
 
 extern "C" int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls) {
   if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
@@ -576,8 +586,8 @@ static int run_allreduce(vr_ctx *ctx, hipStream_t s, const Prepared &p, int tran
     if (used > *advance) *advance = used;
     return VR_OK;
   }
-  hipError_t e = launch_direct_allreduce(s, ctx->dev, t, ctx->nranks, p.a->order, p.in, p.out,
-                                         p.chunk_elems, p.vec_halves);
+  hipError_t e = launch_direct_allreduce(s, ctx->dev, t, ctx->nranks, p.a->order, ctx->dtype, p.in,
+                                         p.out, p.chunk_elems, p.vec_halves);
   if (e != hipSuccess) return fail_hip(e, "launch_direct_allreduce");
   return VR_OK;
 }
@@ -845,8 +855,33 @@ static uint16_t f64_to_f16(double d) {
   return (uint16_t)(sign | bits);
 }
 
+// double -> bfloat16, one rounding (round-to-nearest-even), overflow to infinity.
+static uint16_t f64_to_bf16(double d) {
+  if (d != d) return 0x7fc0;
+  const uint16_t sign = signbit(d) ? 0x8000 : 0;
+  const double a = fabs(d);
+  if (a == 0.0) return sign;
+  if (a >= 0x1.ffp127) return (uint16_t)(sign | 0x7f80);
+  int ex;
+  (void)frexp(a, &ex);
+  int e = ex - 1;
+  if (e < -126) e = -126;
+  const uint32_t q = (uint32_t)nearbyint(ldexp(a, 7 - e));
+  uint32_t bits = (e == -126 && q < 128) ? q : (((uint32_t)(e + 127) << 7) + q - 128);
+  if (bits >= 0x7f80) bits = 0x7f80;
+  return (uint16_t)(sign | bits);
+}
+
+static inline uint16_t f64_to_elem(int dtype, double d) {
+  return dtype == VR_DTYPE_BF16 ? f64_to_bf16(d) : f64_to_f16(d);
+}
+
+extern "C" void vr_fill_pattern_dt(int dtype, uint16_t *host_buf, int rank, size_t n) {
+  for (size_t i = 0; i < n; ++i) host_buf[i] = f64_to_elem(dtype, (double)((int)(i % 32) * (rank + 1)));
+}
+
 extern "C" void vr_fill_pattern(uint16_t *host_buf, int rank, size_t n) {
-  for (size_t i = 0; i < n; ++i) host_buf[i] = f64_to_f16((double)((int)(i % 32) * (rank + 1)));
+  vr_fill_pattern_dt(VR_DTYPE_F16, host_buf, rank, n);
 }
 
 static inline uint64_t splitmix64_at(uint64_t seed, uint64_t k) {
@@ -858,6 +893,11 @@ static inline uint64_t splitmix64_at(uint64_t seed, uint64_t k) {
 
 extern "C" void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dist, double p0,
                             double p1) {
+  vr_generate_dt(VR_DTYPE_F16, host_buf, n, seed, dist, p0, p1);
+}
+
+extern "C" void vr_generate_dt(int dtype, uint16_t *host_buf, size_t n, uint64_t seed, int dist,
+                               double p0, double p1) {
   for (size_t i = 0; i < n; ++i) {
     const uint64_t z0 = splitmix64_at(seed, 2 * (uint64_t)i);
     const uint64_t z1 = splitmix64_at(seed, 2 * (uint64_t)i + 1);
@@ -869,7 +909,7 @@ extern "C" void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dis
       const double u2 = (double)(z1 >> 11) * 0x1.0p-53;
       x = p0 + p1 * (sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2));
     }
-    host_buf[i] = f64_to_f16(x);
+    host_buf[i] = f64_to_elem(dtype, x);
   }
 }
 

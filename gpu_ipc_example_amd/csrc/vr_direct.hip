@@ -62,25 +62,25 @@ __device__ __forceinline__ int operand_rank(int owner, int k) {
 
 // Sum of the N operands in the protocol's association.  The received message is
 // always the left operand of the add (rt64_128.hpp:951-956).
-template <int N, int ORDER, typename V>
+template <int N, int ORDER, int DT, typename V>
 __device__ __forceinline__ V reduce_operands(const V (&x)[N]) {
   if constexpr (ORDER == ORDER_ROTATED) {
     V acc = x[0];
 #pragma unroll
-    for (int k = 1; k < N; ++k) acc = x[k] + acc;
+    for (int k = 1; k < N; ++k) acc = vadd<DT>(x[k], acc);
     return acc;
   } else {
-    V acc = x[1] + x[0];
+    V acc = vadd<DT>(x[1], x[0]);
 #pragma unroll
     for (int k = 2; k < N; k += 2) {
-      const V pair = x[k + 1] + x[k];
-      acc = pair + acc;
+      const V pair = vadd<DT>(x[k + 1], x[k]);
+      acc = vadd<DT>(pair, acc);
     }
     return acc;
   }
 }
 
-template <int N, int ORDER, typename V, int UNROLL, bool NT_LD, bool NT_ST>
+template <int N, int ORDER, int DT, typename V, int UNROLL, bool NT_LD, bool NT_ST>
 __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable out,
                                                            size_t chunk_vecs,
                                                            uint32_t blocks_per_rank) {
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
           x[u][k] = ld<V, NT_LD>(reinterpret_cast<const V *>(src[k] + base_bytes + u * row + lane));
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        const V acc = reduce_operands<N, ORDER, V>(x[u]);
+        const V acc = reduce_operands<N, ORDER, DT, V>(x[u]);
 #pragma unroll
         for (int k = 0; k < N; ++k)
           st<V, NT_ST>(reinterpret_cast<V *>(dst[k] + base_bytes + u * row + lane), acc);
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
 #pragma unroll
           for (int k = 0; k < N; ++k)
             x[0][k] = ld<V, NT_LD>(reinterpret_cast<const V *>(src[k] + base_bytes + u * row + lane));
-          const V acc = reduce_operands<N, ORDER, V>(x[0]);
+          const V acc = reduce_operands<N, ORDER, DT, V>(x[0]);
 #pragma unroll
           for (int k = 0; k < N; ++k)
             st<V, NT_ST>(reinterpret_cast<V *>(dst[k] + base_bytes + u * row + lane), acc);
@@ -234,26 +234,26 @@ static uint32_t blocks_per_rank_for(const DeviceInfo &dev, const Tuning &t, int 
   return (uint32_t)need;
 }
 
-template <int N, int ORDER, typename V, int UNROLL>
+template <int N, int ORDER, int DT, typename V, int UNROLL>
 static hipError_t launch_ar_nt(hipStream_t s, dim3 grid, dim3 block, const Tuning &t,
                                const PtrTable &in, const PtrTable &out, size_t chunk_vecs,
                                uint32_t bpr) {
   if (t.nt_load && t.nt_store)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, V, UNROLL, true, true>), grid, block, 0, s, in,
+    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, true, true>), grid, block, 0, s, in,
                        out, chunk_vecs, bpr);
   else if (t.nt_load)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, V, UNROLL, true, false>), grid, block, 0, s,
+    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, true, false>), grid, block, 0, s,
                        in, out, chunk_vecs, bpr);
   else if (t.nt_store)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, V, UNROLL, false, true>), grid, block, 0, s,
+    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, false, true>), grid, block, 0, s,
                        in, out, chunk_vecs, bpr);
   else
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, V, UNROLL, false, false>), grid, block, 0, s,
+    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, false, false>), grid, block, 0, s,
                        in, out, chunk_vecs, bpr);
   return hipGetLastError();
 }
 
-template <int N, int ORDER, typename V>
+template <int N, int ORDER, int DT, typename V>
 static hipError_t launch_ar_unroll(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
                                    const PtrTable &in, const PtrTable &out, size_t chunk_vecs) {
   const int unroll = (N >= 16) ? 1 : (t.unroll >= 4 && N <= 8 ? 4 : (t.unroll >= 2 ? 2 : 1));
@@ -261,36 +261,40 @@ static hipError_t launch_ar_unroll(hipStream_t s, const DeviceInfo &dev, const T
   const dim3 grid(bpr * N), block(t.block);
   switch (unroll) {
     case 4:
-      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, V, 4>(s, grid, block, t, in, out, chunk_vecs, bpr);
+      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, DT, V, 4>(s, grid, block, t, in, out, chunk_vecs, bpr);
       [[fallthrough]];
     case 2:
-      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, V, 2>(s, grid, block, t, in, out, chunk_vecs, bpr);
+      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, DT, V, 2>(s, grid, block, t, in, out, chunk_vecs, bpr);
       [[fallthrough]];
     default:
-      return launch_ar_nt<N, ORDER, V, 1>(s, grid, block, t, in, out, chunk_vecs, bpr);
+      return launch_ar_nt<N, ORDER, DT, V, 1>(s, grid, block, t, in, out, chunk_vecs, bpr);
   }
 }
 
 template <int N, int ORDER>
-static hipError_t launch_ar_vec(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
+static hipError_t launch_ar_vec(hipStream_t s, const DeviceInfo &dev, const Tuning &t, DType dtype,
                                 const PtrTable &in, const PtrTable &out, size_t chunk_elems,
                                 int vec_halves) {
-  if (vec_halves == 8) return launch_ar_unroll<N, ORDER, h8>(s, dev, t, in, out, chunk_elems / 8);
-  return launch_ar_unroll<N, ORDER, h4>(s, dev, t, in, out, chunk_elems / 4);
+  if (dtype == DT_BF16) {
+    if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_BF16, h8>(s, dev, t, in, out, chunk_elems / 8);
+    return launch_ar_unroll<N, ORDER, DT_BF16, h4>(s, dev, t, in, out, chunk_elems / 4);
+  }
+  if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_F16, h8>(s, dev, t, in, out, chunk_elems / 8);
+  return launch_ar_unroll<N, ORDER, DT_F16, h4>(s, dev, t, in, out, chunk_elems / 4);
 }
 
 hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
-                                   Order order, const PtrTable &in, const PtrTable &out,
+                                   Order order, DType dtype, const PtrTable &in, const PtrTable &out,
                                    size_t chunk_elems, int vec_halves) {
   if (chunk_elems == 0) return hipSuccess;
 #define VR_CASE(NN)                                                                              \
   case NN:                                                                                       \
     if (order == ORDER_BISECT) {                                                                 \
       if constexpr (NN >= 4)                                                                     \
-        return launch_ar_vec<NN, ORDER_BISECT>(s, dev, t, in, out, chunk_elems, vec_halves);     \
+        return launch_ar_vec<NN, ORDER_BISECT>(s, dev, t, dtype, in, out, chunk_elems, vec_halves);     \
       return hipErrorInvalidValue;                                                               \
     }                                                                                            \
-    return launch_ar_vec<NN, ORDER_ROTATED>(s, dev, t, in, out, chunk_elems, vec_halves);
+    return launch_ar_vec<NN, ORDER_ROTATED>(s, dev, t, dtype, in, out, chunk_elems, vec_halves);
   switch (nranks) {
     VR_CASE(2)
     VR_CASE(4)

@@ -15,6 +15,11 @@ struct PtrTable {
   void *p[VR_MAX_RANKS];
 };
 
+enum DType : int {
+  DT_F16 = 0,   // IEEE binary16, added with v_pk_add_f16
+  DT_BF16 = 1,  // bfloat16, added as binary32 and rounded to nearest even (v_cvt_pk_bf16_f32)
+};
+
 enum Order : int {
   ORDER_ROTATED = 0,  // chain from the chunk owner: parallel/sequential/ring/simple transmit
   ORDER_BISECT = 1,   // pair sums, then chain over pairs: BisectPTransmit
@@ -41,7 +46,7 @@ struct DeviceInfo {
 // (16-byte accesses) or 4 (8-byte accesses, for chunks or pointers that are only
 // 8-byte aligned).
 hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
-                                   Order order, const PtrTable &in, const PtrTable &out,
+                                   Order order, DType dtype, const PtrTable &in, const PtrTable &out,
                                    size_t chunk_elems, int vec_halves);
 hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
                                    const PtrTable &in, const PtrTable &out, size_t nelems,
@@ -76,7 +81,23 @@ uint32_t wire_slot_bytes_max();
 // cooperative: hipLaunchCooperativeKernel instead of a plain launch.
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
                        uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
-                       bool cooperative);
+                       bool cooperative, DType dtype);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
+
+
+#ifdef __HIPCC__
+// Element-wise sum of two registers holding 16-bit elements of type DT.  The
+// registers are typed as _Float16 vectors for the memory instructions; bfloat16
+// reinterprets them for the add.
+template <int DT, typename V>
+__device__ __forceinline__ V vadd(V a, V b) {
+  if constexpr (DT == DT_F16) {
+    return a + b;
+  } else {
+    typedef __bf16 B __attribute__((ext_vector_type(sizeof(V) / 2)));
+    return __builtin_bit_cast(V, __builtin_bit_cast(B, a) + __builtin_bit_cast(B, b));
+  }
+}
+#endif
 
 }  // namespace vr

@@ -9,6 +9,7 @@
 //   -r/--ranks N       number of virtual ranks (the MPI world size of the reference)
 //   -t/--transport     direct | wire
 //   -d/--device        HIP device index
+//   --dtype            f16 | bf16 (the reference is built for one test_type, main.cpp:45)
 // Run protocol (main.cpp:48-109): run #1 with `flag`; with -v verify and return;
 // otherwise two more warm-ups (flag+100, flag+150), then the timed run (flag+200)
 // whose kernel time is printed as "[rank] Running time: <ns>ns" for every rank.
@@ -27,7 +28,7 @@
 namespace {
 
 struct Options {
-  std::string nelems = "8MB", algo = "small", transport = "default";
+  std::string nelems = "8MB", algo = "small", transport = "default", dtype = "f16";
   size_t groups = 1, subgroups = 4, flag = 0xe00f100f;
   uint32_t simd = 16;
   bool verify = false, grid_given = false;
@@ -56,7 +57,8 @@ Options parse(int argc, char **argv) {
     if (a == "-h" || a == "--help") {
       printf("usage: vr_main [-n 8MB] [-r 8] [-a small|simple|bisect|parallel|small_ring|simple_ring|"
              "small_pcie|simple_pcie|small_pcie_p|simple_pcie_p|allgather_small|allgather_simple]\n"
-             "               [-g groups -w subgroups -s simd] [-f flag] [-t direct|wire] [-d device] [-v]\n");
+             "               [-g groups -w subgroups -s simd] [-f flag] [-t direct|wire] [-d device]\n"
+             "               [--dtype f16|bf16] [-v]\n");
       exit(0);
     }
     if (take(i, argc, argv, "n", "nelems", &v)) o.nelems = v;
@@ -68,29 +70,44 @@ Options parse(int argc, char **argv) {
     else if (take(i, argc, argv, "r", "ranks", &v)) o.ranks = atoi(v.c_str());
     else if (take(i, argc, argv, "t", "transport", &v)) o.transport = v;
     else if (take(i, argc, argv, "d", "device", &v)) o.device = atoi(v.c_str());
+    else if (take(i, argc, argv, "D", "dtype", &v)) o.dtype = v;
     // the reference ignores what it does not know (allow_unrecognised_options)
   }
   return o;
 }
 
-// Host-side binary16 sum in rank order, like allreduce.cpp:18-27 does on sycl::half.
-// _Float16 arithmetic rounds to nearest even at every assignment.
+// Host-side sum in rank order in the element type, like allreduce.cpp:18-27 does on
+// sycl::half / bfloat16.  _Float16 and __bf16 arithmetic round to nearest even at
+// every assignment.
+int g_dtype = VR_DTYPE_F16;
 uint16_t h_bits(_Float16 h) { uint16_t u; memcpy(&u, &h, 2); return u; }
 _Float16 h_from(uint16_t u) { _Float16 h; memcpy(&h, &u, 2); return h; }
+float bf_to_float(uint16_t u) { uint32_t w = (uint32_t)u << 16; float f; memcpy(&f, &w, 4); return f; }
+uint16_t float_to_bf(float f) {
+  uint32_t w; memcpy(&w, &f, 4);
+  if ((w & 0x7f800000u) == 0x7f800000u && (w & 0x7fffffu)) return (uint16_t)((w >> 16) | 0x40);
+  w += 0x7fffu + ((w >> 16) & 1u);
+  return (uint16_t)(w >> 16);
+}
+double elem_value(uint16_t u) { return g_dtype == VR_DTYPE_BF16 ? (double)bf_to_float(u) : (double)h_from(u); }
+uint16_t elem_add(uint16_t a, uint16_t b) {
+  if (g_dtype == VR_DTYPE_BF16) return float_to_bf(bf_to_float(a) + bf_to_float(b));
+  return h_bits((_Float16)(h_from(a) + h_from(b)));
+}
 
 int verify_allreduce(const std::vector<std::vector<uint16_t>> &got, int world, size_t nelems) {
   std::vector<std::vector<uint16_t>> ranks(world, std::vector<uint16_t>(nelems));
-  for (int r = 0; r < world; ++r) vr_fill_pattern(ranks[r].data(), r, nelems);
+  for (int r = 0; r < world; ++r) vr_fill_pattern_dt(g_dtype, ranks[r].data(), r, nelems);
   size_t printed = 0, bad = 0;
   for (int rank = 0; rank < world; ++rank)
     for (size_t i = 0; i < nelems; ++i) {
-      _Float16 sum = (_Float16)0.0f;
-      for (int r = 0; r < world; ++r) sum = (_Float16)(sum + h_from(ranks[r][i]));
-      if (h_bits(sum) != got[rank][i]) {
+      uint16_t sum = 0;                                   // T sum = 0.0
+      for (int r = 0; r < world; ++r) sum = elem_add(sum, ranks[r][i]);
+      if (sum != got[rank][i]) {
         ++bad;
         if (printed++ < 16)
-          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", (double)sum,
-                 (double)h_from(got[rank][i]), rank, i);
+          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", elem_value(sum),
+                 elem_value(got[rank][i]), rank, i);
       }
     }
   if (bad == 0) printf("verify: %d ranks x %zu elements match the host sum\n", world, nelems);
@@ -100,15 +117,15 @@ int verify_allreduce(const std::vector<std::vector<uint16_t>> &got, int world, s
 
 int verify_allgather(const std::vector<std::vector<uint16_t>> &got, int world, size_t nelems) {
   std::vector<uint16_t> want(nelems * world);
-  for (int r = 0; r < world; ++r) vr_fill_pattern(want.data() + (size_t)r * nelems, r, nelems);
+  for (int r = 0; r < world; ++r) vr_fill_pattern_dt(g_dtype, want.data() + (size_t)r * nelems, r, nelems);
   size_t printed = 0, bad = 0;
   for (int rank = 0; rank < world; ++rank)
     for (size_t i = 0; i < nelems * world; ++i)
       if (want[i] != got[rank][i]) {
         ++bad;
         if (printed++ < 16)
-          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", (double)h_from(want[i]),
-                 (double)h_from(got[rank][i]), rank, i);
+          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", elem_value(want[i]),
+                 elem_value(got[rank][i]), rank, i);
       }
   if (bad == 0) printf("verify: %d ranks x %zu gathered elements match\n", world, nelems * world);
   else printf("verify: %zu mismatches\n", bad);
@@ -129,7 +146,11 @@ int main(int argc, char **argv) try {
   if (o.grid_given && o.subgroups % 4 != 0)
     throw std::logic_error("Subgroup numbers must be multiple of 4");   // main.cpp:289-291
 
+  if (o.dtype == "bf16") g_dtype = VR_DTYPE_BF16;
+  else if (o.dtype != "f16") throw std::invalid_argument("dtype must be f16 or bf16");
+
   vrank::VirtualRanks ranks(world, o.device);
+  ranks.setDtype(g_dtype);
   if (o.transport == "direct") ranks.setTransport(VR_TRANSPORT_DIRECT);
   else if (o.transport == "wire") ranks.setTransport(VR_TRANSPORT_WIRE);
   else if (o.transport != "default") throw std::invalid_argument("transport must be direct or wire");
@@ -139,7 +160,7 @@ int main(int argc, char **argv) try {
   std::vector<uint16_t> host(nelems);
   for (int r = 0; r < world; ++r) {
     vrank::check(vr_malloc(o.device, alloc, &input[r]));
-    vr_fill_pattern(host.data(), r, nelems);
+    vr_fill_pattern_dt(g_dtype, host.data(), r, nelems);
     vrank::check(vr_copy_to_device(input[r], host.data(), alloc));
     if (gather) {
       vrank::check(vr_malloc(o.device, alloc * world, &output[r]));

@@ -55,7 +55,7 @@ struct Spin {
 
 // ---- wire formats ---------------------------------------------------------------
 
-template <int U>
+template <int U, int DT>
 struct WireLL {
   static constexpr uint32_t kWireBytes = 64u * 4u * U;   // payload one wave moves per step
   static constexpr uint32_t kSlotBytes = 64u * 8u * U;   // message bytes in the sink
@@ -83,7 +83,7 @@ struct WireLL {
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const h2 s = __builtin_bit_cast(h2, m.d[u]) + __builtin_bit_cast(h2, v.d[u]);
+      const h2 s = vadd<DT>(__builtin_bit_cast(h2, m.d[u]), __builtin_bit_cast(h2, v.d[u]));
       v.d[u] = __builtin_bit_cast(uint32_t, s);
     }
   }
@@ -125,7 +125,7 @@ struct WireLL {
 // receiver's lane trusts its segment once the segment's flag lane has seen the
 // expected flag (wave vote).  Like the reference's format this rests on a
 // 64-byte segment written by one instruction becoming visible as a whole.
-template <int U>
+template <int U, int DT>
 struct WireLL64 {
   static constexpr uint32_t kWireBytes = 480u * U;
   static constexpr uint32_t kSlotBytes = 512u * U;
@@ -163,7 +163,7 @@ struct WireLL64 {
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int k = 0; k < 2; ++k) {   // the flag lane's second dword is rewritten by send()
-        const h2 s = __builtin_bit_cast(h2, m.d[u][k]) + __builtin_bit_cast(h2, v.d[u][k]);
+        const h2 s = vadd<DT>(__builtin_bit_cast(h2, m.d[u][k]), __builtin_bit_cast(h2, v.d[u][k]));
         v.d[u][k] = __builtin_bit_cast(uint32_t, s);
       }
   }
@@ -204,7 +204,7 @@ struct WireLL64 {
 // flag; the receiver polls the flag word and executes an acquire fence (cache
 // invalidate) before it loads the payload.  Assumes nothing about store
 // atomicity, and pays two cache-maintenance operations per message for it.
-template <int U, typename V>
+template <int U, typename V, int DT>
 struct WireFlag {
   static constexpr uint32_t kWireBytes = 64u * (uint32_t)sizeof(V) * U;
   static constexpr uint32_t kSlotBytes = kWireBytes;
@@ -231,7 +231,7 @@ struct WireFlag {
   }
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) v.d[u] = m.d[u] + v.d[u];
+    for (int u = 0; u < U; ++u) v.d[u] = vadd<DT>(m.d[u], v.d[u]);
   }
   static __device__ __forceinline__ void send(char *slot, uint32_t *flagword, const Reg &v,
                                               uint32_t flag, uint32_t lane) {
@@ -548,27 +548,35 @@ static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 gri
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   switch (fmt) {
-    case WIRE_FMT_LL: return WireLL<kUnrollLL>::kWireBytes;
-    case WIRE_FMT_LL64: return WireLL64<kUnrollLL64>::kWireBytes;
+    case WIRE_FMT_LL: return WireLL<kUnrollLL, DT_F16>::kWireBytes;
+    case WIRE_FMT_LL64: return WireLL64<kUnrollLL64, DT_F16>::kWireBytes;
     default:
-      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8>::kWireBytes
-                             : WireFlag<kUnrollFlag, h4>::kWireBytes;
+      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16>::kWireBytes
+                             : WireFlag<kUnrollFlag, h4, DT_F16>::kWireBytes;
   }
 }
 
-uint32_t wire_slot_bytes_max() { return WireFlag<kUnrollFlag, h8>::kSlotBytes; }
+uint32_t wire_slot_bytes_max() { return WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes; }
+
+template <int DT>
+static hipError_t launch_wire_dt(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves,
+                                 int nranks, dim3 grid, dim3 block, WireArgs &args, bool cooperative) {
+  if (fmt == WIRE_FMT_LL)
+    return launch_flow<WireLL<kUnrollLL, DT>>(s, flow, nranks, grid, block, args, cooperative);
+  if (fmt == WIRE_FMT_LL64)
+    return launch_flow<WireLL64<kUnrollLL64, DT>>(s, flow, nranks, grid, block, args, cooperative);
+  if (vec_halves == 8)
+    return launch_flow<WireFlag<kUnrollFlag, h8, DT>>(s, flow, nranks, grid, block, args, cooperative);
+  return launch_flow<WireFlag<kUnrollFlag, h4, DT>>(s, flow, nranks, grid, block, args, cooperative);
+}
 
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
                        uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
-                       bool cooperative) {
+                       bool cooperative, DType dtype) {
   const dim3 grid(blocks_per_rank * nranks), block(block_threads);
-  if (fmt == WIRE_FMT_LL)
-    return launch_flow<WireLL<kUnrollLL>>(s, flow, nranks, grid, block, args, cooperative);
-  if (fmt == WIRE_FMT_LL64)
-    return launch_flow<WireLL64<kUnrollLL64>>(s, flow, nranks, grid, block, args, cooperative);
-  if (vec_halves == 8)
-    return launch_flow<WireFlag<kUnrollFlag, h8>>(s, flow, nranks, grid, block, args, cooperative);
-  return launch_flow<WireFlag<kUnrollFlag, h4>>(s, flow, nranks, grid, block, args, cooperative);
+  if (dtype == DT_BF16)
+    return launch_wire_dt<DT_BF16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative);
+  return launch_wire_dt<DT_F16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative);
 }
 
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {

@@ -49,6 +49,17 @@ inline void check(int status) {
   }
 }
 
+// ---- element types ---------------------------------------------------------------------
+// The reference instantiates sycl::half and sycl::ext::oneapi::bfloat16
+// (allreduce.cpp:1215-1294).  Any 2-byte T is accepted as binary16 bits; T =
+// vrank::bfloat16 (or a type for which dtype_of is specialised) selects the
+// bfloat16 add.
+struct bfloat16 {
+  std::uint16_t bits;
+};
+template <typename T> struct dtype_of { static constexpr int value = VR_DTYPE_F16; };
+template <> struct dtype_of<bfloat16> { static constexpr int value = VR_DTYPE_BF16; };
+
 // ---- protocol tags -----------------------------------------------------------------
 // Stand-ins for the reference's wire-format classes; only their compile-time
 // constants survive (message size and wire capacity at the given sub-group size).
@@ -137,6 +148,7 @@ class VirtualRanks {
   void setTransport(int transport) { transport_ = transport; }
   int transport() const { return transport_; }
   void setTuning(const char *key, int value) { check(vr_ctx_set_tuning(ctx_, key, value)); }
+  void setDtype(int dtype) { check(vr_ctx_set_dtype(ctx_, dtype)); }
   // Waits for `stream` and reports a wire-transport poll time-out, if any.
   void wait(void *stream = nullptr) { check(vr_ctx_check(ctx_, stream)); }
 
@@ -155,7 +167,7 @@ template <typename T, int NRanks, template <typename, int> class Proto,
           template <typename, int, template <typename, int> class, int> class Transmit,
           int SubGroupSize = 16>
 struct AllReduce {
-  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
   static_assert(detail::allreduce_algo<Proto, Transmit>() >= 0,
                 "this <Proto, Transmit> pair is not one the reference instantiates");
   static_assert(SubGroupSize == 16 || SubGroupSize == 32, "Unsupported Sub-group size");
@@ -181,17 +193,20 @@ struct AllReduce {
 
   // Enqueue on `stream`; in place on the constructor's buffers.
   void operator()(void *stream = nullptr) {
+    ranks_.setDtype(dtype_of<T>::value);
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
   // "construct, then allreduce(stream, inputs, nelems)": run on other buffers of
   // a shape this object was built for.
   void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
+    ranks_.setDtype(dtype_of<T>::value);
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                        &seqNo_));
   }
   void allreduce(void *stream, T *const inputs[], T *const outputs[], std::size_t nelems) {
+    ranks_.setDtype(dtype_of<T>::value);
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)),
                        reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &seqNo_));
@@ -221,7 +236,7 @@ struct AllReduce {
 template <typename T, int NRanks, template <typename, int, int> class Transmit = BisectPTransmit,
           int SubGroupSize = 16>
 struct bisectPAllReduce {
-  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
   static constexpr int algo = VR_ALGO_BISECT;
   static constexpr int BiNRanks = NRanks / 2;
   static constexpr int wireCapacity = 120;
@@ -240,10 +255,12 @@ struct bisectPAllReduce {
     return {g.groups, g.subgroups, (std::uint32_t)SubGroupSize};
   }
   void operator()(void *stream = nullptr) {
+    ranks_.setDtype(dtype_of<T>::value);
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
   void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
+    ranks_.setDtype(dtype_of<T>::value);
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                        &seqNo_));
@@ -269,7 +286,7 @@ template <typename T, int NRanks, template <typename, int> class Proto,
           template <typename, int, template <typename, int> class, int> class Transmit = RingTransmit,
           int SubGroupSize = 16>
 struct AllGather {
-  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
   static_assert(detail::same_transmit<Transmit, RingTransmit>::value &&
                     (detail::same_proto<Proto, Rt64_PCIE>::value ||
                      detail::same_proto<Proto, Rt64_128_PCIE>::value),
@@ -312,10 +329,11 @@ struct AllGather {
 template <typename T>
 void testTransmit(const std::string &transmitType, LaunchParam launchParam, VirtualRanks &ranks,
                   T *const inputs[], std::size_t nelems, std::uint32_t step, void *stream = nullptr) {
-  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
   int algo = -1;
   check(vr_algo_from_string(transmitType.c_str(), &algo));
   if (vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
+  ranks.setDtype(dtype_of<T>::value);
   check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transport(),
                           reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                           step, launchParam.groups, launchParam.subgroups, launchParam.simd));
@@ -325,7 +343,7 @@ template <typename T>
 void testAllgather(const std::string &transmitType, VirtualRanks &ranks, T *const inputs[],
                    T *const outputs[], std::size_t nelems, std::uint32_t &step,
                    void *stream = nullptr) {
-  static_assert(sizeof(T) == 2, "this build moves binary16 elements only");
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
   int algo = -1;
   check(vr_algo_from_string(transmitType.c_str(), &algo));
   if (!vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");

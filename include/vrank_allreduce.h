@@ -86,6 +86,16 @@ typedef enum vr_transport {
   VR_TRANSPORT_WIRE = 2,
 } vr_transport;
 
+/* Element types the reference instantiates (allreduce.cpp:1215-1294: sycl::half and
+ * sycl::ext::oneapi::bfloat16; main.cpp:45 runs bfloat16).  Both are 2 bytes, so
+ * sizes, alignment rules and data movement are identical; only the add differs:
+ * binary16 adds natively, bfloat16 adds as binary32 and rounds the sum to nearest
+ * even.  A context starts as VR_DTYPE_F16. */
+typedef enum vr_dtype {
+  VR_DTYPE_F16 = 0,
+  VR_DTYPE_BF16 = 1,
+} vr_dtype;
+
 typedef struct vr_ctx vr_ctx;
 
 /* ---- lifetime --------------------------------------------------------------- */
@@ -96,6 +106,8 @@ typedef struct vr_ctx vr_ctx;
 int vr_ctx_create(int device, int nranks, vr_ctx **out);
 int vr_ctx_destroy(vr_ctx *ctx);
 int vr_ctx_nranks(const vr_ctx *ctx);
+int vr_ctx_set_dtype(vr_ctx *ctx, int dtype);   /* element type of the following collectives */
+int vr_ctx_get_dtype(const vr_ctx *ctx);
 
 /* ---- validation (host only, no GPU needed) ------------------------------------ */
 
@@ -193,6 +205,10 @@ void vr_fill_pattern(uint16_t *host_buf, int rank, size_t n);     /* utils.hpp:1
 /* Seeded data: dist 0 = uniform [p0,p1), 1 = normal(mean p0, sd p1); splitmix64
  * keyed by seed, element i from draws 2i, 2i+1; rounded once to binary16. */
 void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dist, double p0, double p1);
+/* The same two for either element type. */
+void vr_fill_pattern_dt(int dtype, uint16_t *host_buf, int rank, size_t n);
+void vr_generate_dt(int dtype, uint16_t *host_buf, size_t n, uint64_t seed, int dist, double p0,
+                    double p1);
 /* "8MB" -> 8*1024*1024, "64K", "2G", plain digits (main.cpp:17-34). */
 int vr_parse_nelems(const char *text, size_t *out);
 

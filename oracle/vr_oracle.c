@@ -146,6 +146,22 @@ static inline int is_nan16(uint16_t h) { return (h & 0x7c00) == 0x7c00 && (h & 0
 
 int vro_f16_same(uint16_t a, uint16_t b) { return a == b || (is_nan16(a) && is_nan16(b)); }
 
+/* bfloat16: the upper half of a binary32.  Sum in binary32 (exact inputs, one
+ * rounding), then round to nearest even on the 16 dropped bits; NaN stays NaN. */
+uint16_t vro_bf16_add(uint16_t a, uint16_t b) {
+  uint32_t ua = (uint32_t)a << 16, ub = (uint32_t)b << 16, us;
+  float fa, fb, fs;
+  memcpy(&fa, &ua, 4);
+  memcpy(&fb, &ub, 4);
+  fs = fa + fb;
+  memcpy(&us, &fs, 4);
+  if ((us & 0x7f800000u) == 0x7f800000u && (us & 0x007fffffu)) return (uint16_t)((us >> 16) | 0x0040);
+  us += 0x7fffu + ((us >> 16) & 1u);
+  return (uint16_t)(us >> 16);
+}
+
+static inline int is_nan_bf16(uint16_t h) { return (h & 0x7f80) == 0x7f80 && (h & 0x7f); }
+
 /* Hot inner add for the order loops.  The float route when F16C exists (fast),
  * else the integer route; both give identical bits for non-NaN results. */
 #if defined(__x86_64__)
@@ -215,7 +231,40 @@ static uint16_t f64_to_f16(double d) {
 
 uint16_t vro_f64_to_f16(double d) { return f64_to_f16(d); }
 
+/* double -> bfloat16 with one rounding (8 significant bits, binary32's exponent range). */
+uint16_t vro_f64_to_bf16(double d) {
+  if (d != d) return 0x7fc0;
+  const uint16_t sign = signbit(d) ? 0x8000 : 0;
+  const double a = fabs(d);
+  if (a == 0.0) return sign;
+  if (a >= 0x1.ffp127) return (uint16_t)(sign | 0x7f80);   /* halfway to 2^128 and beyond -> inf */
+  int ex;
+  (void)frexp(a, &ex);
+  int e = ex - 1;
+  if (e < -126) e = -126;                                   /* subnormal grid */
+  const uint32_t q = (uint32_t)nearbyint(ldexp(a, 7 - e)); /* 0..256 */
+  uint32_t bits = (e == -126 && q < 128) ? q : (((uint32_t)(e + 127) << 7) + q - 128);
+  if (bits >= 0x7f80) bits = 0x7f80;
+  return (uint16_t)(sign | bits);
+}
+
+void vro_fill_pattern_dt(int dtype, uint16_t *buf, int rank, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    const double v = (double)((int)(i % 32) * (rank + 1));
+    buf[i] = dtype == VRO_BF16 ? vro_f64_to_bf16(v) : f64_to_f16(v);
+  }
+}
+
+static void generate_impl(int dtype, uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, double p1);
+
 void vro_generate(uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, double p1) {
+  generate_impl(VRO_F16, buf, n, seed, dist, p0, p1);
+}
+void vro_generate_dt(int dtype, uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, double p1) {
+  generate_impl(dtype, buf, n, seed, dist, p0, p1);
+}
+
+static void generate_impl(int dtype, uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, double p1) {
 #pragma omp parallel for schedule(static)
   for (size_t i = 0; i < n; ++i) {
     const uint64_t z0 = splitmix64_at(seed, 2 * (uint64_t)i);
@@ -229,7 +278,7 @@ void vro_generate(uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, d
       const double u2 = (double)(z1 >> 11) * 0x1.0p-53;        /* [0,1) */
       x = p0 + p1 * (sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2));
     }
-    buf[i] = f64_to_f16(x);
+    buf[i] = dtype == VRO_BF16 ? vro_f64_to_bf16(x) : f64_to_f16(x);
   }
 }
 
@@ -307,6 +356,21 @@ __attribute__((target("f16c"))) static void order_hw(int mode, uint16_t *out,
 }
 #endif
 
+static void order_bf16(int mode, uint16_t *out, const uint16_t *const in[], int nranks, size_t n) {
+  ORDER_BODY(vro_bf16_add);
+}
+
+static int order_shape_ok(int mode, int nranks, size_t n);
+
+int vro_allreduce_order_dt(int dtype, int mode, uint16_t *out, const uint16_t *const in[], int nranks,
+                           size_t n) {
+  if (mode < 0 || mode > 2 || !order_shape_ok(mode, nranks, n)) return -2;
+  if (n == 0) return 0;
+  if (dtype == VRO_BF16) order_bf16(mode, out, in, nranks, n);
+  else order_soft(mode, out, in, nranks, n);
+  return 0;
+}
+
 static int order_shape_ok(int mode, int nranks, size_t n) {
   if (nranks < 1 || nranks > MAXR) return 0;
   if (mode == 0) return 1;
@@ -350,6 +414,15 @@ int vro_allreduce_order_soft(int mode, uint16_t *out, const uint16_t *const in[]
 void vro_allgather(uint16_t *out, const uint16_t *const in[], int nranks, size_t n) {
 #pragma omp parallel for schedule(static)
   for (int r = 0; r < nranks; ++r) memcpy(out + (size_t)r * n, in[r], n * sizeof(uint16_t));
+}
+
+size_t vro_count_mismatch_dt(int dtype, const uint16_t *a, const uint16_t *b, size_t n) {
+  size_t bad = 0;
+#pragma omp parallel for schedule(static) reduction(+ : bad)
+  for (size_t i = 0; i < n; ++i)
+    bad += dtype == VRO_BF16 ? !(a[i] == b[i] || (is_nan_bf16(a[i]) && is_nan_bf16(b[i])))
+                             : !vro_f16_same(a[i], b[i]);
+  return bad;
 }
 
 size_t vro_count_mismatch(const uint16_t *a, const uint16_t *b, size_t n) {
@@ -430,11 +503,18 @@ static void store_wire(const wire_fmt *f, uint16_t *dst, const uint32_t *payload
   }
 }
 
-/* v = m + v, element-wise in binary16 (received message is the left operand). */
+/* Element type of the emulators' adds; the *_dt entry points set it for one call.
+ * (The emulators are single-threaded test helpers.) */
+static int g_emul_dtype = VRO_F16;
+static inline uint16_t emul_add(uint16_t a, uint16_t b) {
+  return g_emul_dtype == VRO_BF16 ? vro_bf16_add(a, b) : vro_f16_add_soft(a, b);
+}
+
+/* v = m + v, element-wise in T (received message is the left operand). */
 static void accum(uint32_t *v, const uint32_t *m, int ndw) {
   for (int k = 0; k < ndw; ++k) {
-    const uint16_t lo = vro_f16_add_soft((uint16_t)(m[k] & 0xffff), (uint16_t)(v[k] & 0xffff));
-    const uint16_t hi = vro_f16_add_soft((uint16_t)(m[k] >> 16), (uint16_t)(v[k] >> 16));
+    const uint16_t lo = emul_add((uint16_t)(m[k] & 0xffff), (uint16_t)(v[k] & 0xffff));
+    const uint16_t hi = emul_add((uint16_t)(m[k] >> 16), (uint16_t)(v[k] >> 16));
     v[k] = (uint32_t)lo | ((uint32_t)hi << 16);
   }
 }
@@ -713,5 +793,21 @@ int vro_emulate_bisect(uint16_t *const io[], int nranks, size_t n, int groups, i
     free(gath[r]);
   }
   free(regs);
+  return rc;
+}
+
+int vro_emulate_parallel_dt(int dtype, uint16_t *const io[], int nranks, size_t n, int wire, int groups,
+                            int subgroups, uint32_t seq_no) {
+  g_emul_dtype = dtype;
+  const int rc = vro_emulate_parallel(io, nranks, n, wire, groups, subgroups, seq_no);
+  g_emul_dtype = VRO_F16;
+  return rc;
+}
+
+int vro_emulate_bisect_dt(int dtype, uint16_t *const io[], int nranks, size_t n, int groups,
+                          int subgroups, uint32_t seq_no) {
+  g_emul_dtype = dtype;
+  const int rc = vro_emulate_bisect(io, nranks, n, groups, subgroups, seq_no);
+  g_emul_dtype = VRO_F16;
   return rc;
 }

@@ -127,6 +127,25 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire,
 int vro_emulate_bisect(uint16_t *const io[], int nranks, size_t n,
                        int groups, int subgroups, uint32_t seq_no);
 
+/* ---- bfloat16 (the reference's other instantiated type, allreduce.cpp:1229-1294) ------- *
+ * sycl::ext::oneapi::bfloat16 adds as float and rounds the sum to nearest even;
+ * `dtype` below is VRO_F16 or VRO_BF16 and selects the element arithmetic of the
+ * same order / emulator code.  Pinned by torch.bfloat16 CPU arithmetic on random
+ * and boundary operands, hand cases (256+1, 256+3, overflow to inf) and the
+ * emulator-vs-closed-form agreement. */
+enum { VRO_F16 = 0, VRO_BF16 = 1 };
+uint16_t vro_bf16_add(uint16_t a, uint16_t b);
+uint16_t vro_f64_to_bf16(double d);
+void vro_fill_pattern_dt(int dtype, uint16_t *buf, int rank, size_t n);
+void vro_generate_dt(int dtype, uint16_t *buf, size_t n, uint64_t seed, int dist, double p0, double p1);
+/* mode: 0 rank order, 1 rotated, 2 bisect. */
+int vro_allreduce_order_dt(int dtype, int mode, uint16_t *out, const uint16_t *const in[], int nranks,
+                           size_t n);
+int vro_emulate_parallel_dt(int dtype, uint16_t *const io[], int nranks, size_t n, int wire, int groups,
+                            int subgroups, uint32_t seq_no);
+int vro_emulate_bisect_dt(int dtype, uint16_t *const io[], int nranks, size_t n, int groups,
+                          int subgroups, uint32_t seq_no);
+
 /* ---- host threading for the timed baseline ---------------------------------- */
 /* The order functions are OpenMP-parallel over elements like the reference's
  * host loop; this sets the thread count (0 = leave the runtime's default) and

@@ -146,6 +146,33 @@ static int run_all() {
       EXPECT(b.mismatches(want) == 0);
     }
   }
+  // --- bfloat16 through the same templates -----------------------------------------------------------
+  {
+    VirtualRanks ranks(8);
+    const size_t n = 8 * 4 * 777;
+    std::vector<std::vector<uint16_t>> host(8, std::vector<uint16_t>(n));
+    std::vector<bfloat16 *> dev(8);
+    std::vector<const uint16_t *> hp;
+    for (int r = 0; r < 8; ++r) {
+      vro_generate_dt(VRO_BF16, host[r].data(), n, 91 + r, VRO_DIST_NORMAL, 0.0, 1.0);
+      void *p;
+      check(vr_malloc(0, n * 2, &p));
+      dev[r] = (bfloat16 *)p;
+      check(vr_copy_to_device(p, host[r].data(), n * 2));
+      hp.push_back(host[r].data());
+    }
+    std::vector<uint16_t> want(n), got(n);
+    vro_allreduce_order_dt(VRO_BF16, 2, want.data(), hp.data(), 8, n);
+    uint32_t step = 5;
+    bisectPAllReduce<bfloat16, 8>::launch(ranks, dev.data(), n, step);
+    ranks.wait();
+    for (int r = 0; r < 8; ++r) {
+      check(vr_copy_to_host(got.data(), dev[r], n * 2));
+      EXPECT(memcmp(got.data(), want.data(), n * 2) == 0);
+      vr_free(dev[r]);
+    }
+    ranks.setDtype(VR_DTYPE_F16);
+  }
   // --- the reference's exceptions -------------------------------------------------------------------------
   {
     VirtualRanks ranks(8), two(2);

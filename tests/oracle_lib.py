@@ -17,6 +17,7 @@ SO = os.path.join(ORACLE_DIR, "libvr_oracle.so")
 DIST_UNIFORM, DIST_NORMAL = 0, 1
 WIRE_RT64, WIRE_RT64_128 = 0, 1
 ORDER_RANK, ORDER_ROTATED, ORDER_BISECT = 0, 1, 2
+F16, BF16 = 0, 1
 
 _u16p = C.POINTER(C.c_uint16)
 
@@ -74,6 +75,26 @@ class Oracle:
         L.vro_emulate_bisect.restype = C.c_int
         L.vro_emulate_bisect.argtypes = [C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int, C.c_int,
                                          C.c_uint32]
+        L.vro_bf16_add.restype = C.c_uint16
+        L.vro_bf16_add.argtypes = [C.c_uint16, C.c_uint16]
+        L.vro_f64_to_bf16.restype = C.c_uint16
+        L.vro_f64_to_bf16.argtypes = [C.c_double]
+        L.vro_fill_pattern_dt.restype = None
+        L.vro_fill_pattern_dt.argtypes = [C.c_int, _u16p, C.c_int, C.c_size_t]
+        L.vro_generate_dt.restype = None
+        L.vro_generate_dt.argtypes = [C.c_int, _u16p, C.c_size_t, C.c_uint64, C.c_int, C.c_double,
+                                      C.c_double]
+        L.vro_allreduce_order_dt.restype = C.c_int
+        L.vro_allreduce_order_dt.argtypes = [C.c_int, C.c_int, _u16p, C.POINTER(_u16p), C.c_int,
+                                             C.c_size_t]
+        L.vro_count_mismatch_dt.restype = C.c_size_t
+        L.vro_count_mismatch_dt.argtypes = [C.c_int, _u16p, _u16p, C.c_size_t]
+        L.vro_emulate_parallel_dt.restype = C.c_int
+        L.vro_emulate_parallel_dt.argtypes = [C.c_int, C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int,
+                                              C.c_int, C.c_int, C.c_uint32]
+        L.vro_emulate_bisect_dt.restype = C.c_int
+        L.vro_emulate_bisect_dt.argtypes = [C.c_int, C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int,
+                                            C.c_int, C.c_uint32]
         L.vro_set_threads.restype = C.c_int
         L.vro_set_threads.argtypes = [C.c_int]
 
@@ -135,6 +156,41 @@ class Oracle:
     def count_mismatch(self, a, b):
         assert a.shape == b.shape
         return self.lib.vro_count_mismatch(_ptr(a), _ptr(b), a.size)
+
+    # ---- either element type -----------------------------------------------
+    def fill_pattern_dt(self, dtype, rank, n):
+        a = np.empty(n, np.uint16)
+        self.lib.vro_fill_pattern_dt(dtype, _ptr(a), rank, n)
+        return a
+
+    def generate_dt(self, dtype, n, seed, dist, p0, p1):
+        a = np.empty(n, np.uint16)
+        self.lib.vro_generate_dt(dtype, _ptr(a), n, seed, dist, p0, p1)
+        return a
+
+    def order_dt(self, dtype, mode, ins):
+        n = len(ins[0])
+        out = np.empty(n, np.uint16)
+        rc = self.lib.vro_allreduce_order_dt(dtype, mode, _ptr(out), _ptr_array(ins), len(ins), n)
+        if rc:
+            raise ValueError("oracle rejected the shape (rc=%d)" % rc)
+        return out
+
+    def count_mismatch_dt(self, dtype, a, b):
+        assert a.shape == b.shape
+        return self.lib.vro_count_mismatch_dt(dtype, _ptr(a), _ptr(b), a.size)
+
+    def emulate_parallel_dt(self, dtype, ins, wire, groups, subgroups, seq_no=1):
+        io = [a.copy() for a in ins]
+        rc = self.lib.vro_emulate_parallel_dt(dtype, _ptr_array(io), len(io), len(io[0]), wire, groups,
+                                              subgroups, seq_no)
+        return rc, io
+
+    def emulate_bisect_dt(self, dtype, ins, groups, subgroups, seq_no=1):
+        io = [a.copy() for a in ins]
+        rc = self.lib.vro_emulate_bisect_dt(dtype, _ptr_array(io), len(io), len(io[0]), groups,
+                                            subgroups, seq_no)
+        return rc, io
 
     # ---- emulators (in place on copies) ----------------------------------
     def emulate_parallel(self, ins, wire, groups, subgroups, seq_no=1):

@@ -82,3 +82,19 @@ def test_cli_timed_run_prints_the_reference_lines():
     assert "---------last run------------------" in r.stdout
     for rank in range(8):
         assert "[%d] Running time: " % rank in r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("world,algo", [(2, "small"), (2, "simple"), (2, "simple_ring"),
+                                        (2, "small_pcie"), (8, "allgather_small"), (4, "allgather_simple")])
+def test_cli_verify_bf16(world, algo):
+    """main.cpp:45 builds the reference for bfloat16; the same -v flow here.  -v
+    compares with the reference's rank-order host sum, which for bfloat16 only
+    coincides with the device order while every partial sum of the pattern is
+    exact in 8 bits or the world has two ranks; hence world 2 for the reductions."""
+    for n in (2048, 16384):
+        for t in ("direct", "wire"):
+            r = run([CLI, "-v", "-n", str(n), "-r", str(world), "-a", algo, "--dtype", "bf16", "-t", t],
+                    timeout=60)
+            assert r.returncode == 0, r.stdout
+            assert "Error Compare" not in r.stdout and "match" in r.stdout, (n, t, r.stdout[-300:])
