@@ -308,11 +308,14 @@ static int wire_clear(vr_ctx *c, hipStream_t s) {
 }
 
 // Launches one wire-transport collective.  `user_wires` (0 = automatic) is the
-// number of sub-groups per rank a caller asked for with -g/-w.  Returns through
-// *flags_used how many consecutive flag values the launch consumes.
+// number of sub-groups per rank a caller asked for with -g/-w.  *seq_io is the
+// first flag value the caller proposes; it is replaced by the one actually used
+// (it restarts from 1 when the 32-bit counter would wrap through 0).  Returns
+// through *flags_used how many consecutive flag values the launch consumes.
 static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
-                       const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t seq,
+                       const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t *seq_io,
                        uint32_t user_wires, uint32_t *flags_used) {
+  uint32_t seq = *seq_io;
   if (seq == 0)
     return fail(VR_ERR_INVALID, "sequence number 0 cannot be told from freshly zeroed scratch");
   if (int rc = wire_prepare(c)) return rc;
@@ -337,11 +340,15 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const uint32_t nslot_min = 4;
   *flags_used = (uint32_t)((steps - 1) / nslot_min + 1);
 
-  // Flags must strictly increase on every slot; a different flow or format
-  // re-interprets the sinks, so start those from a clean slate too.
+  // Flags must strictly increase on every slot and never be 0 (the value of
+  // cleared scratch); a different flow or format re-interprets the sinks.  In all
+  // those cases start from a clean slate.
+  const bool wraps = (uint32_t)(seq + *flags_used) < seq;
+  if (wraps) seq = 1;
   const bool moved_back = w.used && (int32_t)(seq - w.next_min_seq) < 0;
-  if (moved_back || (w.used && (w.last_flow != (int)flow || w.last_fmt != (int)fmt)))
+  if (wraps || moved_back || (w.used && (w.last_flow != (int)flow || w.last_fmt != (int)fmt)))
     if (int rc = wire_clear(c, s)) return rc;
+  *seq_io = seq;
 
   WireArgs args;
   memset(&args, 0, sizeof args);
@@ -386,12 +393,12 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   HIP_TRY(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(VR_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", kernels are built for gfx950");
+  HIP_TRY(hipSetDevice(device));
   vr_ctx *c = new vr_ctx;
   c->nranks = nranks;
   c->dev.device = device;
   c->dev.cus = prop.multiProcessorCount;
   snprintf(c->dev.arch, sizeof c->dev.arch, "%s", prop.gcnArchName);
-  HIP_TRY(hipSetDevice(device));
   *out = c;
   return VR_OK;
 }
@@ -574,16 +581,20 @@ static int resolve_transport(const AlgoInfo *a, int transport, int *out) {
   return VR_OK;
 }
 
-// Runs one all-reduce; *advance receives how far the sequence number moves.
+// Runs one all-reduce starting at sequence number `seq_no`; *next_seq receives
+// the sequence number the following launch should start at.
 static int run_allreduce(vr_ctx *ctx, hipStream_t s, const Prepared &p, int transport,
-                         const Tuning &t, uint32_t seq_no, uint32_t user_wires, uint32_t *advance) {
-  *advance = p.geom.steps;          // getLaunchParam: updateSeqNo += nSteps
+                         const Tuning &t, uint32_t seq_no, uint32_t user_wires, uint32_t *next_seq) {
+  uint32_t advance = p.geom.steps;  // getLaunchParam: updateSeqNo += nSteps
+  *next_seq = seq_no + advance;
   if (transport == VR_TRANSPORT_WIRE) {
     uint32_t used = 0;
-    if (int rc = wire_launch(ctx, s, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, seq_no,
+    if (int rc = wire_launch(ctx, s, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, &seq_no,
                              user_wires, &used))
       return rc;
-    if (used > *advance) *advance = used;
+    if (used > advance) advance = used;
+    *next_seq = seq_no + advance;
+    if (*next_seq == 0) *next_seq = 1;
     return VR_OK;
   }
   hipError_t e = launch_direct_allreduce(s, ctx->dev, t, ctx->nranks, p.a->order, ctx->dtype, p.in,
@@ -599,13 +610,12 @@ extern "C" int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, 
   int tr;
   if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
-  const uint32_t start = *seq;
-  uint32_t advance = 0;
+  uint32_t next = *seq;
   if (int rc = run_allreduce(ctx, (hipStream_t)stream, p, tr,
                              tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place),
-                             start, 0, &advance))
+                             *seq, 0, &next))
     return rc;
-  *seq = start + advance;
+  *seq = next;
   return VR_OK;
 }
 
@@ -634,9 +644,9 @@ extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transp
   t.force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
   // Wire transport: groups x subgroups is the number of sub-groups (wires) per rank.
   const uint64_t wires = (uint64_t)groups * subgroups;
-  uint32_t advance = 0;
+  uint32_t next = 0;
   return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no,
-                       wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &advance);
+                       wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &next);
 }
 
 struct PreparedGather {
@@ -688,11 +698,12 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
   if (transport == VR_TRANSPORT_WIRE) {
-    uint32_t used = 0;
-    if (int rc = wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves, *seq,
+    uint32_t used = 0, start = *seq;
+    if (int rc = wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start,
                              0, &used))
       return rc;
-    *seq += used > p.geom.steps ? used : p.geom.steps;
+    *seq = start + (used > p.geom.steps ? used : p.geom.steps);
+    if (*seq == 0) *seq = 1;
     return VR_OK;
   }
   if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
@@ -763,10 +774,9 @@ extern "C" int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transp
   const Tuning t = tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place);
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
-    const uint32_t start = ctx->seq_no;
-    uint32_t advance = 0;
-    int rc = run_allreduce(ctx, s, p, tr, t, start, 0, &advance);
-    ctx->seq_no = start + advance;
+    uint32_t next = ctx->seq_no;
+    int rc = run_allreduce(ctx, s, p, tr, t, ctx->seq_no, 0, &next);
+    ctx->seq_no = next;
     return rc;
   });
 }
@@ -781,9 +791,10 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
     if (transport == VR_TRANSPORT_WIRE) {
-      uint32_t used = 0;
-      int rc = wire_launch(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, ctx->seq_no, 0, &used);
-      ctx->seq_no += used > p.geom.steps ? used : p.geom.steps;
+      uint32_t used = 0, start = ctx->seq_no;
+      int rc = wire_launch(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start, 0, &used);
+      ctx->seq_no = start + (used > p.geom.steps ? used : p.geom.steps);
+      if (ctx->seq_no == 0) ctx->seq_no = 1;
       return rc;
     }
     hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);

@@ -132,6 +132,27 @@ def test_sequence_number_moving_backwards_is_safe(ctxs, oracle):
     assert e.value.code == "INVALID"
 
 
+def test_sequence_number_wrap_never_uses_flag_zero(ctxs, oracle):
+    """A 32-bit counter that would run through 0 restarts from 1 on clean scratch."""
+    import ctypes as C
+    ctx = ctxs[8]
+    n = 8 * 4096 * 8
+    ins = H.make_inputs(oracle, 8, n, 88)
+    want = oracle.rotated(ins)
+    ctx.seq_no = C.c_uint32(0xFFFFFFFF)
+    for _ in range(3):
+        got, _ = H.run_allreduce(ctx, "simple", ins, transport=WIRE)
+        H.assert_all_ranks_equal(oracle, got, want)
+        assert ctx.seq_no.value != 0
+    assert ctx.seq_no.value < 1000
+    src = H.RankBuffers(8, n)
+    src.upload(ins)
+    ctx.allreduce_grid("small", src.ptrs, n, 8, 8, 16, transport=WIRE, seq_no=0xFFFFFFFF)
+    ctx.check()
+    H.assert_all_ranks_equal(oracle, src.download(), want)
+    src.free()
+
+
 def test_poll_timeout_is_reported_and_recoverable(ctxs, oracle):
     """A spin limit of one poll makes some wave give up before its message has
     arrived; every wave still runs to completion, the context reports the
