@@ -127,36 +127,36 @@ def hbm_ceilings(binding, ctx):
     return out
 
 
-def verify(name, host, ins, outs):
-    """Bit-exact check of the buffers against the CPU oracle (checker only)."""
+def cpu_leg(name, gpu_results, budget_s):
+    """The CPU side of the run, and the only place that touches the oracle: time
+    its OpenMP loop for this workload on the host cores (a reported baseline),
+    and use its output as the checker for what the GPU produced on the same
+    inputs.  `gpu_results` maps a workload name to the per-rank output arrays of
+    one GPU launch on fresh inputs."""
     from tests import oracle_lib
     o = oracle_lib.load()
-    n, algo, ne, *_ = WORKLOADS[name]
-    if algo.startswith("allgather"):
-        want = o.allgather(host)
-    elif algo == "bisect":
-        want = o.bisect(host)
-    else:
-        want = o.rotated(host)
-    bad = 0
-    for b in (outs if outs else ins):
-        bad += o.count_mismatch(b.download(np.uint16, len(want)), want)
-    return bad
 
+    def reference(wname):
+        n, algo, ne, dist, p0, p1, seed = WORKLOADS[wname]
+        host = [o.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
+        fn = (o.allgather if algo.startswith("allgather")
+              else (o.bisect if algo == "bisect" else o.rotated))
+        return host, fn
 
-def cpu_baseline(name, budget_s):
-    """The oracle's OpenMP loop for this workload on the host cores (reported only)."""
-    from tests import oracle_lib
-    o = oracle_lib.load()
-    n, algo, ne, dist, p0, p1, seed = WORKLOADS[name]
-    host = [o.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
-    fn = o.allgather if algo.startswith("allgather") else (o.bisect if algo == "bisect" else o.rotated)
-    out = {}
-    for label, threads in (("all", 0), ("one", 1)):
-        used = o.set_threads(threads if threads else (os.cpu_count() or 1))
-        if threads == 0:
+    mismatches = {}
+    for wname, outs in gpu_results.items():
+        host, fn = reference(wname)
+        want = fn(host)
+        mismatches[wname] = int(sum(o.count_mismatch(g, want) for g in outs))
+
+    host, fn = reference(name)
+    timing = {}
+    for label in ("all", "one"):
+        if label == "all":
             env = os.environ.get("OMP_NUM_THREADS")
             used = o.set_threads(int(env) if env else min(os.cpu_count() or 1, 64))
+        else:
+            used = o.set_threads(1)
         fn(host)                                          # warm-up, page faults
         best, reps, t_start = 1e30, 0, time.perf_counter()
         while True:
@@ -164,17 +164,17 @@ def cpu_baseline(name, budget_s):
             fn(host)
             dt = time.perf_counter() - t0
             best, reps = min(best, dt), reps + 1
-            if reps >= 5 and time.perf_counter() - t_start > budget_s / 2:
+            elapsed = time.perf_counter() - t_start
+            if (reps >= 5 and elapsed > budget_s / 4) or elapsed > budget_s / 2:
                 break
-            if time.perf_counter() - t_start > budget_s:
-                break
-        out[label] = (algorithmic_bytes(name) / best / 1e9, used, reps, best)
-    gb_all, cores, reps, best = out["all"]
-    return {
+        timing[label] = (algorithmic_bytes(name) / best / 1e9, used, reps, best)
+    gb_all, cores, reps, best = timing["all"]
+    baseline = {
         "value": round(gb_all, 3), "unit": "GB/s", "cores": cores, "kind": "port",
         "sample": "%s full size, best of %d passes (%.1f ms); 1 thread: %.3f GB/s" % (
-            name, reps, best * 1e3, out["one"][0]),
+            name, reps, best * 1e3, timing["one"][0]),
     }
+    return baseline, mismatches
 
 
 def sweep(vr, binding, args):
@@ -294,10 +294,14 @@ def main():
         k, v = kv.split("=")
         ctx.set_tuning(**{k: int(v)})
 
-    # correctness of exactly this configuration, on fresh inputs
+    # one launch of exactly this configuration on fresh inputs, kept for the checker
+    want_check = not args.no_cpu and not args.only_headline
+    gpu_results = {}
     launch(ctx, name, *sets[0])
     ctx.sync()
-    mismatches = verify(name, host, *sets[0])
+    if want_check:
+        count = (n * ne) if algo.startswith("allgather") else ne
+        gpu_results[name] = [b.download(np.uint16, count) for b in (sets[0][1] or sets[0][0])]
     if args.inplace:
         for b, a in zip(sets[0][0], host):
             b.upload(a)
@@ -332,7 +336,7 @@ def main():
                                len(sets), len(sets) * (B if not args.inplace else B / 2) / 2**20)
                            if len(sets) > 1 else "every step reuses one buffer set (cache-warm)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-        "bit_exact_vs_oracle": mismatches == 0, "mismatches": int(mismatches),
+        "bit_exact_vs_oracle": None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
@@ -357,21 +361,26 @@ def main():
         c2, h2, s2 = setup(vr, binding, "cfg2", True, 1)
         launch(c2, "cfg2", *s2[0])
         c2.sync()
-        bad2 = verify("cfg2", h2, *s2[0])
+        if want_check:
+            gpu_results["cfg2"] = [b.download(np.uint16, WORKLOADS["cfg2"][2]) for b in s2[0][0]]
         time_kernels(binding, c2, "cfg2", s2, 50)
         lat = time_kernels(binding, c2, "cfg2", s2, args.latency_iters) * 1e3
         p50 = float(np.percentile(lat, 50))
         result["latency_1MiB_per_rank"] = {
             "workload": describe("cfg2") + ", in place", "iters": args.latency_iters,
             "p50_us": round(p50, 3), "p99_us": round(float(np.percentile(lat, 99)), 3),
-            "min_us": round(float(lat.min()), 3), "bit_exact_vs_oracle": bad2 == 0,
+            "min_us": round(float(lat.min()), 3), "bit_exact_vs_oracle": None,
             "GBps_at_p50": round(algorithmic_bytes("cfg2") / (p50 * 1e-6) / 1e9, 1),
             "note": "one HIP event pair per launch: includes ~2 us of event overhead that a "
                     "kernel trace does not show; buffers are cache-resident"}
         result["hbm_ceilings"] = hbm_ceilings(binding, ctx)
 
-    if not args.no_cpu and not args.only_headline:
-        result["cpu_baseline"] = cpu_baseline(name, args.cpu_seconds)
+    if want_check:
+        result["cpu_baseline"], bad = cpu_leg(name, gpu_results, args.cpu_seconds)
+        result["bit_exact_vs_oracle"] = bad[name] == 0
+        result["mismatches"] = bad[name]
+        if "cfg2" in bad and "latency_1MiB_per_rank" in result:
+            result["latency_1MiB_per_rank"]["bit_exact_vs_oracle"] = bad["cfg2"] == 0
     print(json.dumps(result, default=float))
 
 
