@@ -209,7 +209,7 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 // User overrides of the launch heuristics; -1 = let the library decide.
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
-  int wire_fenced = -1, wire_cooperative = -1;
+  int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1;
 };
 
 // Scratch of the wire transport: per virtual rank one scatter and one gather
@@ -239,6 +239,7 @@ struct vr_ctx {
 };
 
 static const uint32_t kDefaultSpinLimit = 1u << 22;
+static const int kWireBlocksPerCu = 2;
 
 static void wire_free(vr_ctx *c) {
   WireState &w = c->wire;
@@ -269,13 +270,20 @@ static int wire_allocate(vr_ctx *c) {
   WireState &w = c->wire;
   HIP_TRY(hipSetDevice(c->dev.device));
   const int N = c->nranks;
-  // One work-group per CU keeps every wire of every rank co-resident.
-  w.blocks_per_rank_max = (uint32_t)(c->dev.cus / N);
+  // A few 256-lane work-groups per CU (default one; a CU holds eight of them)
+  // keep every wire of every rank co-resident.
+  const int per_cu = c->tune.wire_blocks_per_cu > 0 ? c->tune.wire_blocks_per_cu : kWireBlocksPerCu;
+  w.blocks_per_rank_max = (uint32_t)(c->dev.cus * per_cu / N);
   if (w.blocks_per_rank_max == 0) w.blocks_per_rank_max = 1;
-  const uint32_t wpr_max = w.blocks_per_rank_max * (w.block_threads / 64);
-  const size_t entries = (size_t)N * wpr_max + 2 * (size_t)N;
-  w.sink_bytes = entries * kWireMaxSlots * wire_slot_bytes_max();
-  w.flag_bytes = entries * kWireMaxSlots * sizeof(uint32_t);
+  const size_t wpr_max = (size_t)w.blocks_per_rank_max * (w.block_threads / 64);
+  // Slots a sink must hold: ring / sequential / all-gather index [peer][wire] with
+  // 4 slots each; parallel indexes [wire + rank] and bisect [close wires + N/2 |
+  // far wires], both with 8 slots.
+  const size_t slots_ring = 4 * (size_t)N * wpr_max;
+  const size_t slots_flat = (size_t)kWireMaxSlots * (2 * wpr_max + (size_t)N);
+  const size_t slots = slots_ring > slots_flat ? slots_ring : slots_flat;
+  w.sink_bytes = slots * wire_slot_bytes_max();
+  w.flag_bytes = slots * sizeof(uint32_t);
   for (int r = 0; r < N; ++r) {
     HIP_TRY(hipMalloc(&w.scatter[r], w.sink_bytes));
     HIP_TRY(hipMalloc(&w.gather[r], w.sink_bytes));
@@ -437,6 +445,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "oneshot")) return &ctx->tune.oneshot;
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
+  if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
   return nullptr;
 }
 
@@ -454,6 +463,10 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
          !strcmp(key, "wire_fenced") || !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
+    if (!strcmp(key, "wire_blocks_per_cu")) {
+      if (value < 1 || value > 4) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be in [1,4]");
+      if (ctx->wire.ready) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be set before the first wire-transport launch");
+    }
   }
   *f = value;
   return VR_OK;
