@@ -12,6 +12,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
 CPP_TEST = os.path.join(ROOT, "tests", "cpp", "test_host_api")
+GRAPH_TEST = os.path.join(ROOT, "tests", "cpp", "test_graph")
 
 
 def run(cmd, **kw):
@@ -47,6 +48,15 @@ def test_header_compiles_with_plain_gxx(tmp_path):
         "int main() { return 0; }\n")
     r = run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-I", os.path.join(ROOT, "include"), str(src)])
     assert r.returncode == 0, r.stdout
+
+
+@pytest.mark.gpu
+def test_direct_transport_replays_correctly_from_a_hip_graph():
+    """A captured small -> copy -> bisect sequence, replayed six times with eager
+    work and synchronisation in between; every replay is compared with the oracle."""
+    assert os.path.exists(GRAPH_TEST), "run make -C tests/cpp"
+    r = run([GRAPH_TEST], timeout=120)
+    assert r.returncode == 0 and "graph ok" in r.stdout, r.stdout
 
 
 @pytest.mark.gpu
