@@ -15,7 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libvrank_allreduce.so")
 
 ALGOS = ("small", "simple", "bisect", "parallel", "small_pcie_p", "simple_pcie_p", "small_ring",
-         "simple_ring", "small_pcie", "simple_pcie", "allgather_small", "allgather_simple")
+         "simple_ring", "small_pcie", "simple_pcie", "allgather_small", "allgather_simple",
+         "simple_transmit")
 TRANSPORT_DEFAULT, TRANSPORT_DIRECT, TRANSPORT_WIRE = 0, 1, 2
 
 # vr_status -> Python exception class; the texts come from vr_strerror.

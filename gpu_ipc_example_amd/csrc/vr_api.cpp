@@ -59,7 +59,7 @@ extern "C" const char *vr_version(void) { return "vrank_allreduce 0.1 (gfx950)";
 // algorithm table
 // ---------------------------------------------------------------------------------
 
-enum TransmitKind { T_PARALLEL, T_BISECT, T_RING, T_SEQUENTIAL };
+enum TransmitKind { T_PARALLEL, T_BISECT, T_RING, T_SEQUENTIAL, T_SIMPLE };
 
 struct AlgoInfo {
   const char *name;
@@ -75,6 +75,7 @@ struct AlgoInfo {
       case T_BISECT: return WIRE_BISECT;
       case T_RING: return WIRE_RING;
       case T_SEQUENTIAL: return WIRE_SEQUENTIAL;
+      case T_SIMPLE: return WIRE_SIMPLE;
       default: return WIRE_PARALLEL;
     }
   }
@@ -98,6 +99,7 @@ static const AlgoInfo kAlgos[VR_ALGO_COUNT_] = {
     {"simple_pcie", T_SEQUENTIAL, 16, 240, false, ORDER_ROTATED, false},
     {"allgather_small", T_RING, 16, 128, true, ORDER_ROTATED, true},
     {"allgather_simple", T_RING, 16, 240, true, ORDER_ROTATED, false},
+    {"simple_transmit", T_SIMPLE, 8, 120, false, ORDER_ROTATED, false},
 };
 
 static const AlgoInfo *algo_info(int algo) {
@@ -281,7 +283,10 @@ static int wire_allocate(vr_ctx *c) {
   // far wires], both with 8 slots.
   const size_t slots_ring = 4 * (size_t)N * wpr_max;
   const size_t slots_flat = (size_t)kWireMaxSlots * (2 * wpr_max + (size_t)N);
-  const size_t slots = slots_ring > slots_flat ? slots_ring : slots_flat;
+  // SimpleTransmit: one 2 MiB ring section per sender.
+  const size_t slots_simple = (size_t)N * (kSimpleSectionBytes / wire_slot_bytes_max());
+  size_t slots = slots_ring > slots_flat ? slots_ring : slots_flat;
+  if (slots_simple > slots) slots = slots_simple;
   w.sink_bytes = slots * wire_slot_bytes_max();
   w.flag_bytes = slots * sizeof(uint32_t);
   for (int r = 0; r < N; ++r) {
@@ -342,11 +347,16 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   size_t want = user_wires ? (size_t)user_wires / psg * psg : wires_per_chunk * psg;
   if (want < psg) want = psg;
   if (want > wpr_limit) want = wpr_limit;
+  // SimpleTransmit's ring sections hold 2 MiB of messages per sender; a sender
+  // runs at most one step ahead of its receivers, so two steps must fit.
+  const size_t per_section = kSimpleSectionBytes / wire_slot_bytes_max();
+  if (flow == WIRE_SIMPLE && want > per_section / 2) want = per_section / 2;
   const uint32_t wpr = (uint32_t)want;
   const uint32_t blocks_per_rank = (uint32_t)div_up(wpr, waves_per_block);
   const size_t steps = div_up(wires_per_chunk, wpr / psg);
   const uint32_t nslot_min = 4;
-  *flags_used = (uint32_t)((steps - 1) / nslot_min + 1);
+  *flags_used = flow == WIRE_SIMPLE ? (uint32_t)(steps * wpr / per_section + 1)
+                                    : (uint32_t)((steps - 1) / nslot_min + 1);
 
   // Flags must strictly increase on every slot and never be 0 (the value of
   // cleared scratch); a different flow or format re-interprets the sinks.  In all

@@ -57,7 +57,8 @@ hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, vo
 
 
 // Wire transport ------------------------------------------------------------------
-enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER };
+enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER, WIRE_SIMPLE };
+constexpr uint32_t kSimpleSectionBytes = 0x200000;   // simple_transmit.hpp:11
 enum WireFormat : int {
   WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
   WIRE_FMT_LL64 = 1,  // 60 B payload + 4 B flag per 64-byte segment (Rt64_128 family)

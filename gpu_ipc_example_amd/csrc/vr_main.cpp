@@ -56,7 +56,7 @@ Options parse(int argc, char **argv) {
     if (a == "-v" || a == "--verify") { o.verify = true; continue; }
     if (a == "-h" || a == "--help") {
       printf("usage: vr_main [-n 8MB] [-r 8] [-a small|simple|bisect|parallel|small_ring|simple_ring|"
-             "small_pcie|simple_pcie|small_pcie_p|simple_pcie_p|allgather_small|allgather_simple]\n"
+             "small_pcie|simple_pcie|small_pcie_p|simple_pcie_p|simple_transmit|allgather_small|allgather_simple]\n"
              "               [-g groups -w subgroups -s simd] [-f flag] [-t direct|wire] [-d device]\n"
              "               [--dtype f16|bf16] [-v]\n");
       exit(0);

@@ -6,8 +6,8 @@
 // into peers' scatter/gather sinks in device scratch, polls its own sinks, adds
 // in the reference's order and stores.  Sink indexing, slot rotation and flag
 // values follow parallel_transmit.hpp:47-58,75,93-122, sequential_transmit.hpp:
-// 57-81,112-206 (Sequential), 262-278,333-516 (Ring) and bisect_transmit.hpp:
-// 286-424,432-481, re-tiled for 64-lane wavefronts.
+// 57-81,112-206 (Sequential), 262-278,333-516 (Ring), simple_transmit.hpp:16-179
+// and bisect_transmit.hpp:286-424,432-481, re-tiled for 64-lane wavefronts.
 //
 // Three wire formats:
 //   WireLL    (Rt64 family, rt64.hpp:334-341): every 8-byte store carries 4 bytes
@@ -363,6 +363,58 @@ __global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
   }
 }
 
+// ---- SimpleTransmit (simple_transmit.hpp:16-179) ---------------------------------------------
+// The older three-phase form: scatter / pollRecvReduceBcast / pollGatherOutputs.
+// Same data flow as the sequential transmit, but the sinks are linear rings: each
+// sender owns one 2 MiB section of every peer's sink, a message lands at
+// ringOffset = transmitted bytes % section, and the flag counts how often the
+// ring has wrapped (seqNo + transmitted bytes / section).
+template <int N, typename W>
+__global__ __launch_bounds__(1024) void k_wire_simple(WireArgs a) {
+  constexpr uint32_t kSection = 0x200000;
+  constexpr uint32_t kPerSection = kSection / W::kSlotBytes;
+  VR_WAVE_PROLOGUE;
+  const uint32_t wpr = a.waves_per_rank;
+  const char *src = static_cast<const char *>(a.in.p[r]);
+  char *dst = static_cast<char *>(a.out.p[r]);
+  auto sink = [&](void *base, int section, uint32_t pos) {
+    return static_cast<char *>(base) + (size_t)section * kSection + (size_t)pos * W::kSlotBytes;
+  };
+  auto flagw = [&](void *base, int section, uint32_t pos) {
+    return static_cast<uint32_t *>(base) + (size_t)section * kPerSection + pos;
+  };
+  size_t t = 0;
+  for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
+    const size_t message = t * wpr + wid;                         // sinkOffset / wireTransSize
+    const uint32_t pos = (uint32_t)(message % kPerSection);       // ringOffset
+    const uint32_t flag = a.seq + (uint32_t)(message / kPerSection);   // seqNo + seqDelta
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    for (int i = 0; i < N - 1; ++i) {                             // scatter
+      const int next = (r + i + 1) % N;
+      const typename W::Reg p = W::load(src + next * chunk + off, left, lane);
+      W::send(sink(a.scatter.p[next], r, pos), flagw(a.sflag.p[next], r, pos), p, flag, lane);
+    }
+    typename W::Reg v = W::load(src + r * chunk + off, left, lane);    // pollRecvReduceBcast
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      typename W::Reg m;
+      W::recv(sink(a.scatter.p[r], next, pos), flagw(a.sflag.p[r], next, pos), m, flag, lane, spin);
+      W::add(v, m);
+    }
+    W::store(dst + r * chunk + off, left, lane, v);               // write back locally first
+    for (int i = 0; i < N - 1; ++i) {
+      const int next = (r + i + 1) % N;
+      W::send(sink(a.gather.p[next], r, pos), flagw(a.gflag.p[next], r, pos), v, flag, lane);
+    }
+    for (int i = 0; i < N - 1; ++i) {                             // pollGatherOutputs
+      const int next = (r + i + 1) % N;
+      typename W::Reg m;
+      W::recv(sink(a.gather.p[r], next, pos), flagw(a.gflag.p[r], next, pos), m, flag, lane, spin);
+      W::store(dst + next * chunk + off, left, lane, m);
+    }
+  }
+}
+
 // ---- RingTransmit::runAllreduce (sequential_transmit.hpp:429-472) ----------------------------
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
@@ -522,6 +574,7 @@ static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 gri
     switch (flow) {                                                                         \
       case WIRE_PARALLEL: fn = reinterpret_cast<const void *>(&k_wire_parallel<NN, W>); break;   \
       case WIRE_SEQUENTIAL: fn = reinterpret_cast<const void *>(&k_wire_sequential<NN, W>); break; \
+      case WIRE_SIMPLE: fn = reinterpret_cast<const void *>(&k_wire_simple<NN, W>); break;         \
       case WIRE_RING: fn = reinterpret_cast<const void *>(&k_wire_ring<NN, W>); break;           \
       case WIRE_ALLGATHER: fn = reinterpret_cast<const void *>(&k_wire_allgather<NN, W>); break;  \
       case WIRE_BISECT:                                                                     \

@@ -66,6 +66,8 @@ typedef enum vr_algo {
   VR_ALGO_SIMPLE_PCIE = 9,      /* Rt64_128_PCIE + SequentialTransmit */
   VR_ALGO_ALLGATHER_SMALL = 10, /* Rt64_PCIE     + RingTransmit::runAllgather */
   VR_ALGO_ALLGATHER_SIMPLE = 11,/* Rt64_128_PCIE + RingTransmit::runAllgather */
+  VR_ALGO_SIMPLE_TRANSMIT = 12, /* Rt64_128 + SimpleTransmit (simple_transmit.hpp; has no -a string
+                                   in the reference, whose include of it is disabled) */
   VR_ALGO_COUNT_
 } vr_algo;
 

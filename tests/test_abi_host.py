@@ -37,6 +37,7 @@ def test_algo_strings():
     assert vr.lib().vr_algo_message_bytes(vr.algo_id("small")) == 8
     assert vr.lib().vr_algo_message_bytes(vr.algo_id("simple_ring")) == 16
     assert vr.lib().vr_algo_is_allgather(vr.algo_id("allgather_small")) == 1
+    assert vr.algo_id("simple_transmit") == 12 and vr.launch_geometry("simple_transmit", 2, 16384) == (3, 64, 1)
 
 
 def test_error_texts_are_the_reference_ones():

@@ -11,7 +11,7 @@ from tests import vr_helpers as H
 
 pytestmark = pytest.mark.gpu
 
-ALGOS8 = ("small", "simple", "bisect", "parallel")
+ALGOS8 = ("small", "simple", "bisect", "parallel", "simple_transmit")
 ALGOS16 = ("small_pcie_p", "simple_pcie_p", "small_ring", "simple_ring", "small_pcie", "simple_pcie")
 
 

@@ -30,7 +30,7 @@ def per_chunk(out, nranks):
 
 
 @pytest.mark.parametrize("algo", ["small", "simple", "parallel", "bisect", "small_ring", "simple_ring",
-                                  "small_pcie", "simple_pcie"])
+                                  "small_pcie", "simple_pcie", "simple_transmit"])
 def test_kat_n8(ctxs, algo):
     ins = [np.full(1024, h(v), np.uint16) for v in (2048, 0, 1, 0, 1, 0, 0, 0)]
     got, _ = H.run_allreduce(ctxs[8], algo, ins, transport=WIRE)
@@ -95,7 +95,7 @@ def test_many_launches_reuse_slots_and_flags(ctxs, oracle):
     from gpu_ipc_example_amd.binding import DeviceBuffer
     ctx = ctxs[8]
     n = 8 * 4096 * 6            # several steps per launch at the automatic grid
-    for algo in ("small", "simple", "bisect", "small_ring", "simple_pcie"):
+    for algo in ("small", "simple", "bisect", "small_ring", "simple_pcie", "simple_transmit"):
         base = H.make_inputs(oracle, 8, n, 900)
         cur = [a.copy() for a in base]
         bufs = [DeviceBuffer(n * 2) for _ in range(8)]
@@ -250,7 +250,20 @@ def test_plain_launch_instead_of_cooperative(oracle):
     ctx.close()
 
 
-@pytest.mark.parametrize("algo", ["simple", "bisect", "simple_ring", "small"])
+def test_simple_transmit_ring_sections_wrap(ctxs, oracle):
+    """Enough messages per sender to run through the 2 MiB ring sections several
+    times in one launch (flag = seqNo + wraps), with small and large grids."""
+    n = 8 * (6 << 20) // 2                        # 6 MiB per rank-chunk, 48 MiB per rank
+    ins = H.make_inputs(oracle, 8, n, 6300)
+    want = oracle.rotated(ins)
+    for grid in (None, (2, 4, 16), (64, 64, 16)):
+        got, _ = H.run_allreduce(ctxs[8], "simple_transmit", ins, transport=WIRE, grid=grid)
+        assert oracle.count_mismatch(got[0], want) == 0, grid
+        for r in range(1, 8):
+            assert oracle.count_mismatch(got[r], got[0]) == 0, (grid, r)
+
+
+@pytest.mark.parametrize("algo", ["simple", "bisect", "simple_ring", "small", "simple_transmit"])
 def test_embedded_flag_formats_under_repetition(ctxs, oracle, algo):
     """Many launches over the same sinks: every 64-byte segment (Rt64_128 family)
     and every 8-byte message (Rt64 family) must arrive whole every time."""

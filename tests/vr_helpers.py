@@ -7,7 +7,7 @@ from gpu_ipc_example_amd.binding import DeviceBuffer
 from tests.oracle_lib import DIST_NORMAL, DIST_UNIFORM
 
 ROTATED_ALGOS = ("small", "simple", "small_pcie_p", "simple_pcie_p", "small_ring", "simple_ring",
-                 "small_pcie", "simple_pcie")
+                 "small_pcie", "simple_pcie", "simple_transmit")
 
 
 def make_inputs(oracle, nranks, n, seed, dist=DIST_NORMAL, p0=0.0, p1=1.0):
