@@ -90,6 +90,7 @@ def lib():
         "vr_time_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_copy": (i, [vp, vp, vp, vp, sz, i, C.POINTER(C.c_float)]),
         "vr_stream_probe": (i, [vp, vp, i, vp, vp, sz]),
+        "vr_probe_xcc_ids": (i, [vp, u32, C.POINTER(u32)]),
         "vr_fill_pattern": (None, [C.POINTER(C.c_uint16), i, sz]),
         "vr_generate": (None, [C.POINTER(C.c_uint16), sz, C.c_uint64, i, C.c_double, C.c_double]),
         "vr_parse_nelems": (i, [C.c_char_p, C.POINTER(sz)]),
@@ -293,6 +294,11 @@ class VirtualRanks:
         """mode: 0 copy, 1 read only, 2 write only."""
         _check(lib().vr_stream_probe(self._h, stream, mode, C.c_void_p(int(dst)),
                                      C.c_void_p(int(src)), nbytes))
+
+    def xcc_ids(self, blocks):
+        out = (C.c_uint32 * blocks)()
+        _check(lib().vr_probe_xcc_ids(self._h, blocks, out))
+        return np.frombuffer(out, np.uint32).copy()
 
     def time_copy(self, dst, src, nbytes, iters, stream=None):
         ms = (C.c_float * iters)()

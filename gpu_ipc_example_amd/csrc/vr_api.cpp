@@ -857,6 +857,17 @@ extern "C" int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, c
   return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
 }
 
+extern "C" int vr_probe_xcc_ids(vr_ctx *ctx, uint32_t blocks, uint32_t *ids_host) {
+  if (!ids_host || blocks == 0 || blocks > 65536) return fail(VR_ERR_INVALID, "bad argument");
+  if (int rc = use_device(ctx)) return rc;
+  uint32_t *d = nullptr;
+  HIP_TRY(hipMalloc((void **)&d, (size_t)blocks * 4));
+  hipError_t e = launch_xcc_probe(nullptr, blocks, d);
+  if (e == hipSuccess) e = hipMemcpy(ids_host, d, (size_t)blocks * 4, hipMemcpyDeviceToHost);
+  (void)hipFree(d);
+  return e == hipSuccess ? VR_OK : fail_hip(e, "xcc probe");
+}
+
 extern "C" int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes,
                             int iters, float *ms_out) {
   Tuning t;

@@ -56,6 +56,8 @@ hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, vo
                        const void *src, size_t bytes, int mode = 0);
 
 
+hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device);
+
 // Wire transport ------------------------------------------------------------------
 enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER, WIRE_SIMPLE };
 constexpr uint32_t kSimpleSectionBytes = 0x200000;   // simple_transmit.hpp:11

@@ -203,6 +203,12 @@ int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t b
 enum { VR_PROBE_COPY = 0, VR_PROBE_READ = 1, VR_PROBE_WRITE = 2 };
 int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, const void *src, size_t bytes);
 
+/* Diagnostic: launches `blocks` work-groups and reports the XCD each one ran on
+ * (ids_host[b]).  The direct kernels give work-group b to virtual rank b % N and
+ * count on the hardware placing it on XCD b % 8, so that with 8 ranks every XCD
+ * serves exactly one rank's chunk.  Synchronous. */
+int vr_probe_xcc_ids(vr_ctx *ctx, uint32_t blocks, uint32_t *ids_host);
+
 /* ---- host helpers -------------------------------------------------------------- */
 
 void vr_fill_pattern(uint16_t *host_buf, int rank, size_t n);     /* utils.hpp:15-19 */

@@ -291,3 +291,10 @@ def test_allgather_rejections(ctxs, oracle):
     with pytest.raises(vr.VRError) as e:
         run_allgather(ctxs[4], "allgather_small", ins)
     assert e.value.code == "UNEVEN"
+
+
+def test_work_groups_land_on_xcd_block_mod_8(ctxs):
+    """The rank-to-XCD affinity the direct kernels are laid out for: work-group b
+    of a launch runs on XCD b % 8 (so each XCD serves one of 8 virtual ranks)."""
+    ids = ctxs[8].xcc_ids(2048)
+    assert (ids == np.arange(2048) % 8).all(), ids[:32]
