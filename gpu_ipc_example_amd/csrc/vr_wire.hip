@@ -113,6 +113,29 @@ struct WireLL {
       if (spin.give_up(polls)) return false;
     }
   }
+  // M messages at once: all loads are in flight together, so the wait costs one
+  // memory round trip instead of M.  Re-polls everything until all have arrived.
+  template <int M>
+  static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
+                                                   const uint32_t *const (&)[M], Reg (&v)[M],
+                                                   uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint64_t msg = __hip_atomic_load(
+              reinterpret_cast<const uint64_t *>(slot[i]) + u * 64 + lane, __ATOMIC_RELAXED, VR_AGENT);
+          v[i].d[u] = (uint32_t)msg;
+          ok = ok && (uint32_t)(msg >> 32) == flag;
+        }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
 };
 
 // Rt64_128 re-tiled for wavefronts (rt64_128.hpp:538-553, 635-685, 724-802): the
@@ -196,6 +219,29 @@ struct WireLL64 {
       if (spin.give_up(polls)) return false;
     }
   }
+  template <int M>
+  static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
+                                                   const uint32_t *const (&)[M], Reg (&v)[M],
+                                                   uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    const bool flag_lane = (lane & 7u) == 7u;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint64_t msg = __hip_atomic_load(
+              reinterpret_cast<const uint64_t *>(slot[i]) + u * 64 + lane, __ATOMIC_RELAXED, VR_AGENT);
+          v[i].d[u][0] = (uint32_t)msg;
+          v[i].d[u][1] = (uint32_t)(msg >> 32);
+          ok = ok && (!flag_lane || v[i].d[u][1] == flag);
+        }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
 };
 
 // Flag-word format: full 16-byte-per-lane payload lines plus ONE flag word per
@@ -253,6 +299,28 @@ struct WireFlag {
     for (int u = 0; u < U; ++u) v.d[u] = reinterpret_cast<const V *>(slot)[u * 64 + lane];
     return true;
   }
+  // M messages: wait for every flag word, ONE acquire fence, then all payloads.
+  template <int M>
+  static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
+                                                   const uint32_t *const (&flagword)[M], Reg (&v)[M],
+                                                   uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+        ok = ok && __hip_atomic_load(flagword[i], __ATOMIC_RELAXED, VR_AGENT) == flag;
+      if (ok) break;                       // same words in every lane: wave-uniform
+      if (spin.give_up(polls)) return false;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[i].d[u] = reinterpret_cast<const V *>(slot[i])[u * 64 + lane];
+    return true;
+  }
 };
 
 // ---- sinks --------------------------------------------------------------------------
@@ -308,12 +376,18 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
       W::send(sk.scat(y, x_id + r, s), sk.sflag(y, x_id + r, s), v, flag, lane);
       W::recv(sk.gath(r, x_id + y, s), sk.gflag(r, x_id + y, s), v, flag, lane, spin);
     } else {                                         // wait, reduce, broadcast
+      const char *ms[N - 1];
+      const uint32_t *mf[N - 1];
+      typename W::Reg m[N - 1];
+#pragma unroll
       for (int i = 0; i < N - 1; ++i) {
         const int next = (r + i + 1) % N;
-        typename W::Reg m;
-        W::recv(sk.scat(r, x_id + next, s), sk.sflag(r, x_id + next, s), m, flag, lane, spin);
-        W::add(v, m);
+        ms[i] = sk.scat(r, x_id + next, s);
+        mf[i] = sk.sflag(r, x_id + next, s);
       }
+      W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+      for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);    // peers in order rank+1, rank+2, ...
       for (int i = 0; i < N - 1; ++i) {
         const int next = (r + i + 1) % N;
         W::send(sk.gath(next, x_id + r, s), sk.gflag(next, x_id + r, s), v, flag, lane);
@@ -343,23 +417,33 @@ __global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
       W::send(sk.scat(next, r * wpr + wid, s), sk.sflag(next, r * wpr + wid, s), p, flag, lane);
     }
     typename W::Reg v = W::load(src + r * chunk + off, left, lane);
+    const char *ms[N - 1];
+    const uint32_t *mf[N - 1];
+    typename W::Reg m[N - 1];
+#pragma unroll
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      typename W::Reg m;
-      W::recv(sk.scat(r, next * wpr + wid, s), sk.sflag(r, next * wpr + wid, s), m, flag, lane, spin);
-      W::add(v, m);
+      ms[i] = sk.scat(r, next * wpr + wid, s);
+      mf[i] = sk.sflag(r, next * wpr + wid, s);
     }
+    W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+    for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);      // peers in order rank+1, rank+2, ...
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
       W::send(sk.gath(next, r * wpr + wid, s), sk.gflag(next, r * wpr + wid, s), v, flag, lane);
     }
     W::store(dst + r * chunk + off, left, lane, v);
+#pragma unroll
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      typename W::Reg m;
-      W::recv(sk.gath(r, next * wpr + wid, s), sk.gflag(r, next * wpr + wid, s), m, flag, lane, spin);
-      W::store(dst + next * chunk + off, left, lane, m);
+      ms[i] = sk.gath(r, next * wpr + wid, s);
+      mf[i] = sk.gflag(r, next * wpr + wid, s);
     }
+    W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+    for (int i = 0; i < N - 1; ++i)
+      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i]);
   }
 }
 
@@ -395,23 +479,33 @@ __global__ __launch_bounds__(1024) void k_wire_simple(WireArgs a) {
       W::send(sink(a.scatter.p[next], r, pos), flagw(a.sflag.p[next], r, pos), p, flag, lane);
     }
     typename W::Reg v = W::load(src + r * chunk + off, left, lane);    // pollRecvReduceBcast
+    const char *ms[N - 1];
+    const uint32_t *mf[N - 1];
+    typename W::Reg m[N - 1];
+#pragma unroll
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      typename W::Reg m;
-      W::recv(sink(a.scatter.p[r], next, pos), flagw(a.sflag.p[r], next, pos), m, flag, lane, spin);
-      W::add(v, m);
+      ms[i] = sink(a.scatter.p[r], next, pos);
+      mf[i] = flagw(a.sflag.p[r], next, pos);
     }
+    W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+    for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);
     W::store(dst + r * chunk + off, left, lane, v);               // write back locally first
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
       W::send(sink(a.gather.p[next], r, pos), flagw(a.gflag.p[next], r, pos), v, flag, lane);
     }
+#pragma unroll
     for (int i = 0; i < N - 1; ++i) {                             // pollGatherOutputs
       const int next = (r + i + 1) % N;
-      typename W::Reg m;
-      W::recv(sink(a.gather.p[r], next, pos), flagw(a.gflag.p[r], next, pos), m, flag, lane, spin);
-      W::store(dst + next * chunk + off, left, lane, m);
+      ms[i] = sink(a.gather.p[r], next, pos);
+      mf[i] = flagw(a.gflag.p[r], next, pos);
     }
+    W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+    for (int i = 0; i < N - 1; ++i)
+      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i]);
   }
 }
 
@@ -528,12 +622,18 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
       W::send(sk.scat(owner, wg + l, s), sk.sflag(owner, wg + l, s), v, flag, lane);
       W::recv(sk.gath(r, wg + y, s), sk.gflag(r, wg + y, s), v, flag, lane, spin);
     } else {
+      const char *ms[B - 1];
+      const uint32_t *mf[B - 1];
+      typename W::Reg m[B - 1];
+#pragma unroll
       for (int i = 0; i < B - 1; ++i) {
         const int l_next = (l + i + 1) % B;
-        typename W::Reg m;
-        W::recv(sk.scat(r, wg + l_next, s), sk.sflag(r, wg + l_next, s), m, flag, lane, spin);
-        W::add(v, m);
+        ms[i] = sk.scat(r, wg + l_next, s);
+        mf[i] = sk.sflag(r, wg + l_next, s);
       }
+      W::template recv_many<B - 1>(ms, mf, m, flag, lane, spin);
+#pragma unroll
+      for (int i = 0; i < B - 1; ++i) W::add(v, m[i]);    // pair sums in order l+1, l+2, ...
       for (int i = 0; i < B - 1; ++i) {
         const int nx = (r + i * 2 + 2) % N;
         W::send(sk.gath(nx, wg + l, s), sk.gflag(nx, wg + l, s), v, flag, lane);
