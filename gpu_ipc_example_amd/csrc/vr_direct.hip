@@ -215,8 +215,8 @@ __global__ __launch_bounds__(1024) void k_probe(h8 *dst, const h8 *src, size_t v
 }
 
 // Records which XCD (accelerator complex die) each work-group of a launch ran on:
-// the rank-to-XCD affinity of the kernels above rests on work-group b landing
-// on XCD b % 8.
+// the rank-to-XCD affinity of the kernels above rests on consecutive work-groups
+// being dealt to consecutive XCDs.
 __global__ void k_xcc_ids(uint32_t *out) {
   if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20);  // XCC_ID[3:0]
 }

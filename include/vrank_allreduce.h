@@ -205,8 +205,9 @@ int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, const void *
 
 /* Diagnostic: launches `blocks` work-groups and reports the XCD each one ran on
  * (ids_host[b]).  The direct kernels give work-group b to virtual rank b % N and
- * count on the hardware placing it on XCD b % 8, so that with 8 ranks every XCD
- * serves exactly one rank's chunk.  Synchronous. */
+ * count on the hardware dealing consecutive work-groups to consecutive XCDs
+ * (XCD (b + s) % 8, s = wherever the previous launch stopped), so that within a
+ * launch of 8 ranks every XCD serves exactly one rank's chunk.  Synchronous. */
 int vr_probe_xcc_ids(vr_ctx *ctx, uint32_t blocks, uint32_t *ids_host);
 
 /* ---- host helpers -------------------------------------------------------------- */

@@ -293,8 +293,11 @@ def test_allgather_rejections(ctxs, oracle):
     assert e.value.code == "UNEVEN"
 
 
-def test_work_groups_land_on_xcd_block_mod_8(ctxs):
-    """The rank-to-XCD affinity the direct kernels are laid out for: work-group b
-    of a launch runs on XCD b % 8 (so each XCD serves one of 8 virtual ranks)."""
-    ids = ctxs[8].xcc_ids(2048)
-    assert (ids == np.arange(2048) % 8).all(), ids[:32]
+def test_work_groups_are_dealt_round_robin_over_the_xcds(ctxs):
+    """The rank-to-XCD affinity the direct kernels are laid out for: consecutive
+    work-groups of a launch go to consecutive XCDs (starting wherever the previous
+    launch stopped), so within a launch each XCD serves exactly one of 8 ranks."""
+    for _ in range(3):
+        ids = ctxs[8].xcc_ids(2048).astype(np.int64)
+        assert ids.min() == 0 and ids.max() == 7
+        assert (((ids - ids[0]) % 8) == np.arange(2048) % 8).all(), ids[:32]
