@@ -211,6 +211,7 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 // User overrides of the launch heuristics; -1 = let the library decide.
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
+  int segment_kib = -1;
   int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1;
 };
 
@@ -453,6 +454,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "nt_load")) return &ctx->tune.nt_load;
   if (!strcmp(key, "nt_store")) return &ctx->tune.nt_store;
   if (!strcmp(key, "oneshot")) return &ctx->tune.oneshot;
+  if (!strcmp(key, "segment_kib")) return &ctx->tune.segment_kib;
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
@@ -469,10 +471,14 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
     if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
       return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
-    if ((!strcmp(key, "nt_load") || !strcmp(key, "nt_store") || !strcmp(key, "oneshot") ||
-         !strcmp(key, "wire_fenced") || !strcmp(key, "wire_cooperative")) &&
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") ||
+         !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
+    if (!strcmp(key, "nt_store") && (value < 0 || value > 2))
+      return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
+    if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))
+      return fail(VR_ERR_INVALID, "segment_kib must be in [1, 1048576]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
       if (value < 1 || value > 4) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be in [1,4]");
       if (ctx->wire.ready) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be set before the first wire-transport launch");
@@ -547,6 +553,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   if (o.nt_load != -1) t.nt_load = o.nt_load;
   if (o.nt_store != -1) t.nt_store = o.nt_store;
   if (o.oneshot != -1) t.oneshot = o.oneshot;
+  if (o.segment_kib != -1) t.segment_bytes = (size_t)o.segment_kib << 10;
   return t;
 }
 
@@ -844,6 +851,7 @@ static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, Tu
   if (o.unroll != -1) d.unroll = o.unroll;
   if (o.nt_load != -1) d.nt_load = o.nt_load;
   if (o.nt_store != -1) d.nt_store = o.nt_store;
+  if (o.segment_kib != -1) d.segment_bytes = (size_t)o.segment_kib << 10;
   *t = d;
   return VR_OK;
 }

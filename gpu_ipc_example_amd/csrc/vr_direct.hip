@@ -13,6 +13,13 @@
 // Per 16-byte column a lane issues N independent dwordx4 loads, N-1 packed
 // binary16 adds per half2, and N dwordx4 stores; nothing is staged in LDS
 // because no datum is used twice.
+//
+// Memory is addressed through buffer resources (one per rank and direction,
+// built in scalar registers from the chunk's base pointer and byte length): a
+// lane supplies a 32-bit byte offset, the hardware drops every access at or
+// beyond the length, so the last tile of a chunk needs no predicate (the
+// reference predicates its tail wire per lane, rt64_128.hpp:570-582), and the
+// cache-policy bits of each access are chosen per launch.
 
 #include "vr_internal.h"
 
@@ -20,21 +27,37 @@ namespace vr {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-template <typename V, bool NT>
-__device__ __forceinline__ V ld(const V *p) {
-  if constexpr (NT)
-    return __builtin_nontemporal_load(p);
-  else
-    return *p;
+// Cache-policy operand of the buffer instructions (gfx940 encoding): bit 0 = sc0,
+// bit 1 = nt, bit 4 = sc1.
+constexpr int kAuxCached = 0;
+constexpr int kAuxStream = 2;            // nt: streaming, do not keep in L2
+constexpr int kAuxStreamAgent = 2 | 16;  // nt sc1: streaming store written through at agent scope
+
+constexpr int load_aux(int nt) { return nt ? kAuxStream : kAuxCached; }
+constexpr int store_aux(int nt) { return nt == 2 ? kAuxStreamAgent : nt == 1 ? kAuxStream : kAuxCached; }
+
+// Raw buffer over [p, p + bytes): stride 0, 32-bit data format word for gfx9.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
 }
 
-template <typename V, bool NT>
-__device__ __forceinline__ void st(V *p, V v) {
-  if constexpr (NT)
-    __builtin_nontemporal_store(v, p);
+template <typename V, int AUX>
+__device__ __forceinline__ V ld(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  if constexpr (sizeof(V) == 16)
+    return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, AUX));
   else
-    *p = v;
+    return __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, AUX));
+}
+
+template <typename V, int AUX>
+__device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, uint32_t off, V v) {
+  if constexpr (sizeof(V) == 16)
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, off, 0, AUX);
+  else
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, off, 0, AUX);
 }
 
 // Rank whose input is the k-th operand of the chain for the chunk owned by
@@ -80,137 +103,103 @@ __device__ __forceinline__ V reduce_operands(const V (&x)[N]) {
   }
 }
 
-template <int N, int ORDER, int DT, typename V, int UNROLL, bool NT_LD, bool NT_ST>
+// One launch covers bytes [seg_off, seg_off + seg_bytes) of every chunk;
+// chunk_pitch is the full chunk length (the distance between chunk starts).
+template <int N, int ORDER, int DT, typename V, int UNROLL, int LD_AUX, int ST_AUX>
 __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable out,
-                                                           size_t chunk_vecs,
+                                                           size_t chunk_pitch, size_t seg_off,
+                                                           uint32_t seg_bytes,
                                                            uint32_t blocks_per_rank) {
   const int owner = blockIdx.x % N;
   const uint32_t jblock = blockIdx.x / N;
-  const int chunk = chunk_of_owner<N, ORDER>(owner);
-  const size_t chunk_base = (size_t)chunk * chunk_vecs;
+  const size_t base = (size_t)chunk_of_owner<N, ORDER>(owner) * chunk_pitch + seg_off;
 
-  // Uniform (scalar) byte pointers to this chunk in every rank's buffer; a lane
-  // adds only its own 32-bit byte offset, so every access is
-  // "global_load/store_dwordx4 v, v_lane, s[base]" and no 64-bit vector address
-  // arithmetic is needed.
-  const char *src[N];
-  char *dst[N];
+  __amdgpu_buffer_rsrc_t src[N], dst[N];
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    src[k] = static_cast<const char *>(in.p[operand_rank<N, ORDER>(owner, k)]) + chunk_base * sizeof(V);
-    dst[k] = static_cast<char *>(out.p[k]) + chunk_base * sizeof(V);
+    src[k] = make_rsrc(static_cast<const char *>(in.p[operand_rank<N, ORDER>(owner, k)]) + base, seg_bytes);
+    dst[k] = make_rsrc(static_cast<char *>(out.p[k]) + base, seg_bytes);
   }
   const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
   const uint32_t row = blockDim.x * (uint32_t)sizeof(V);       // bytes one unroll step spans
-
-  const size_t tile = (size_t)blockDim.x * UNROLL;
-  const size_t stride = tile * blocks_per_rank;
-  for (size_t base = (size_t)jblock * tile; base < chunk_vecs; base += stride) {
+  const uint32_t tile = row * UNROLL;
+  const uint32_t stride = tile * blocks_per_rank;
+  for (uint32_t t = jblock * tile; t < seg_bytes; t += stride) {
     V x[UNROLL][N];
-    const size_t base_bytes = base * sizeof(V);
-    if (base + tile <= chunk_vecs) {
-      // Whole tile in range: UNROLL*N loads in flight with no predication.
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < N; ++k)
-          x[u][k] = ld<V, NT_LD>(reinterpret_cast<const V *>(src[k] + base_bytes + u * row + lane));
+      for (int k = 0; k < N; ++k) x[u][k] = ld<V, LD_AUX>(src[k], t + u * row + lane);
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const V acc = reduce_operands<N, ORDER, DT, V>(x[u]);
+    for (int u = 0; u < UNROLL; ++u) {
+      const V acc = reduce_operands<N, ORDER, DT, V>(x[u]);
 #pragma unroll
-        for (int k = 0; k < N; ++k)
-          st<V, NT_ST>(reinterpret_cast<V *>(dst[k] + base_bytes + u * row + lane), acc);
-      }
-    } else {
-      // Tail tile of the chunk: per-lane predicate, like the reference's tail wire.
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        if (base + (size_t)u * blockDim.x + threadIdx.x < chunk_vecs) {
-#pragma unroll
-          for (int k = 0; k < N; ++k)
-            x[0][k] = ld<V, NT_LD>(reinterpret_cast<const V *>(src[k] + base_bytes + u * row + lane));
-          const V acc = reduce_operands<N, ORDER, DT, V>(x[0]);
-#pragma unroll
-          for (int k = 0; k < N; ++k)
-            st<V, NT_ST>(reinterpret_cast<V *>(dst[k] + base_bytes + u * row + lane), acc);
-        }
-      }
+      for (int k = 0; k < N; ++k) st<V, ST_AUX>(dst[k], t + u * row + lane, acc);
     }
   }
 }
 
 // All-gather: the groups of rank p read p's slice once and store it into slot p
 // of every rank's output (allgather.hpp:79-100 collapsed to one hop).
-template <int N, typename V, int UNROLL, bool NT_LD, bool NT_ST>
+template <int N, typename V, int UNROLL, int LD_AUX, int ST_AUX>
 __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable out,
-                                                           size_t slice_vecs,
+                                                           size_t slice_pitch, size_t seg_off,
+                                                           uint32_t seg_bytes,
                                                            uint32_t blocks_per_rank) {
   const int p = blockIdx.x % N;
   const uint32_t jblock = blockIdx.x / N;
-  const V *src = reinterpret_cast<const V *>(in.p[p]);
-  V *dst[N];
+  const char *src_ptr = static_cast<const char *>(in.p[p]) + seg_off;
+  const __amdgpu_buffer_rsrc_t src = make_rsrc(src_ptr, seg_bytes);
+  __amdgpu_buffer_rsrc_t dst[N];
+  bool skip[N];
 #pragma unroll
-  for (int r = 0; r < N; ++r) dst[r] = reinterpret_cast<V *>(out.p[r]) + (size_t)p * slice_vecs;
-
-  const size_t tile = (size_t)blockDim.x * UNROLL;
-  const size_t stride = tile * blocks_per_rank;
-  for (size_t base = (size_t)jblock * tile; base < slice_vecs; base += stride) {
+  for (int r = 0; r < N; ++r) {
+    char *d = static_cast<char *>(out.p[r]) + (size_t)p * slice_pitch + seg_off;
+    // The reference skips the store when a rank's input already is its own
+    // output slot (sequential_transmit.hpp:496-497).
+    skip[r] = d == src_ptr;
+    dst[r] = make_rsrc(d, seg_bytes);
+  }
+  const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
+  const uint32_t row = blockDim.x * (uint32_t)sizeof(V);
+  const uint32_t tile = row * UNROLL;
+  const uint32_t stride = tile * blocks_per_rank;
+  for (uint32_t t = jblock * tile; t < seg_bytes; t += stride) {
     V x[UNROLL];
-    size_t idx[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      idx[u] = base + (size_t)u * blockDim.x + threadIdx.x;
-      if (idx[u] < slice_vecs) x[u] = ld<V, NT_LD>(src + idx[u]);
-    }
+    for (int u = 0; u < UNROLL; ++u) x[u] = ld<V, LD_AUX>(src, t + u * row + lane);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      if (idx[u] < slice_vecs) {
+    for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-        for (int r = 0; r < N; ++r) {
-          // The reference skips the store when a rank's input already is its
-          // own output slot (sequential_transmit.hpp:496-497).
-          if (reinterpret_cast<const V *>(dst[r]) != src) st<V, NT_ST>(dst[r] + idx[u], x[u]);
-        }
-      }
-    }
+      for (int r = 0; r < N; ++r)
+        if (!skip[r]) st<V, ST_AUX>(dst[r], t + u * row + lane, x[u]);
   }
 }
 
-// Streaming yardsticks: MODE 0 copies, 1 only reads (the sum is kept alive by a
-// store that never executes for finite data), 2 only writes.
-template <int MODE, int UNROLL, bool NT>
-__global__ __launch_bounds__(1024) void k_probe(h8 *dst, const h8 *src, size_t vecs) {
-  const size_t tile = (size_t)blockDim.x * UNROLL;
-  const size_t stride = tile * gridDim.x;
+// Streaming yardsticks over one segment: MODE 0 copies, 1 only reads (the sum is
+// kept alive by a store that never executes for finite data), 2 only writes.
+template <int MODE, int UNROLL, int LD_AUX, int ST_AUX>
+__global__ __launch_bounds__(1024) void k_probe(char *dst_ptr, const char *src_ptr, uint32_t seg_bytes) {
+  const __amdgpu_buffer_rsrc_t src = make_rsrc(src_ptr, seg_bytes);
+  const __amdgpu_buffer_rsrc_t dst = make_rsrc(dst_ptr, seg_bytes);
+  const uint32_t lane = threadIdx.x * 16u, row = blockDim.x * 16u;
+  const uint32_t tile = row * UNROLL, stride = tile * gridDim.x;
   h8 acc = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (size_t base = (size_t)blockIdx.x * tile; base < vecs; base += stride) {
-    const size_t first = base + threadIdx.x;
-    if (base + tile <= vecs) {
-      h8 x[UNROLL];
-      if constexpr (MODE != 2) {
+  for (uint32_t t = blockIdx.x * tile; t < seg_bytes; t += stride) {
+    h8 x[UNROLL];
+    if constexpr (MODE != 2) {
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) x[u] = ld<h8, NT>(src + first + (size_t)u * blockDim.x);
-      }
+      for (int u = 0; u < UNROLL; ++u) x[u] = ld<h8, LD_AUX>(src, t + u * row + lane);
+    }
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        if constexpr (MODE == 0) st<h8, NT>(dst + first + (size_t)u * blockDim.x, x[u]);
-        if constexpr (MODE == 1) acc = acc + x[u];
-        if constexpr (MODE == 2) st<h8, NT>(dst + first + (size_t)u * blockDim.x, acc);
-      }
-    } else {
-      for (int u = 0; u < UNROLL; ++u) {
-        const size_t i = first + (size_t)u * blockDim.x;
-        if (i < vecs) {
-          if constexpr (MODE == 0) st<h8, NT>(dst + i, ld<h8, NT>(src + i));
-          if constexpr (MODE == 1) acc = acc + ld<h8, NT>(src + i);
-          if constexpr (MODE == 2) st<h8, NT>(dst + i, acc);
-        }
-      }
+    for (int u = 0; u < UNROLL; ++u) {
+      if constexpr (MODE == 0) st<h8, ST_AUX>(dst, t + u * row + lane, x[u]);
+      if constexpr (MODE == 1) acc = acc + x[u];
+      if constexpr (MODE == 2) st<h8, ST_AUX>(dst, t + u * row + lane, acc);
     }
   }
   if constexpr (MODE == 1) {
-    if (acc[0] == (_Float16)12345.0f && acc[7] == (_Float16)-321.0f) dst[0] = acc;
+    if (acc[0] == (_Float16)12345.0f && acc[7] == (_Float16)-321.0f) st<h8, kAuxCached>(dst, 0, acc);
   }
 }
 
@@ -228,11 +217,19 @@ hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device
 
 // ---- host-side launch plumbing -------------------------------------------------
 
+// A launch addresses each chunk with 32-bit byte offsets, so longer chunks are
+// covered by several launches of at most Tuning::segment_bytes per chunk.
+static size_t segment_of(const Tuning &t) {
+  size_t seg = t.segment_bytes - t.segment_bytes % 16;
+  if (seg == 0) seg = 16;
+  return seg > (1ull << 30) ? (1ull << 30) : seg;
+}
+
 static uint32_t blocks_per_rank_for(const DeviceInfo &dev, const Tuning &t, int nranks,
-                                    size_t vecs_per_rank, int unroll) {
-  const size_t tile = (size_t)t.block * unroll;
-  size_t need = (vecs_per_rank + tile - 1) / tile;
-  if (need == 0) need = 1;
+                                    size_t bytes_per_rank, size_t tile_bytes) {
+  size_t tiles = (bytes_per_rank + tile_bytes - 1) / tile_bytes;
+  if (tiles == 0) tiles = 1;
+  size_t need = tiles;
   if (t.force_blocks_per_rank) {
     need = t.force_blocks_per_rank;
   } else if (!t.oneshot) {
@@ -242,63 +239,79 @@ static uint32_t blocks_per_rank_for(const DeviceInfo &dev, const Tuning &t, int 
     if (cap == 0) cap = 1;
     if (need > cap) need = cap;
   }
-  if (need > 0x7fffffffu / (size_t)nranks) need = 0x7fffffffu / (size_t)nranks;
+  if (need > tiles) need = tiles;   // a block without a tile has nothing to do
   return (uint32_t)need;
 }
 
+// Calls f(std::integral_constant<int, load aux>, std::integral_constant<int, store aux>)
+// for the launch's cache policies.
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
+
+template <typename F>
+static hipError_t with_policy(const Tuning &t, F &&f) {
+  const int ld_nt = t.nt_load ? 1 : 0;
+  const int st_nt = t.nt_store < 0 ? 0 : (t.nt_store > 2 ? 2 : t.nt_store);
+#define VR_POLICY(L, S) \
+  if (ld_nt == L && st_nt == S) return f(IntC<load_aux(L)>(), IntC<store_aux(S)>());
+  VR_POLICY(0, 0) VR_POLICY(0, 1) VR_POLICY(0, 2) VR_POLICY(1, 0) VR_POLICY(1, 1) VR_POLICY(1, 2)
+#undef VR_POLICY
+  return hipErrorInvalidValue;
+}
+
 template <int N, int ORDER, int DT, typename V, int UNROLL>
-static hipError_t launch_ar_nt(hipStream_t s, dim3 grid, dim3 block, const Tuning &t,
-                               const PtrTable &in, const PtrTable &out, size_t chunk_vecs,
-                               uint32_t bpr) {
-  if (t.nt_load && t.nt_store)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, true, true>), grid, block, 0, s, in,
-                       out, chunk_vecs, bpr);
-  else if (t.nt_load)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, true, false>), grid, block, 0, s,
-                       in, out, chunk_vecs, bpr);
-  else if (t.nt_store)
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, false, true>), grid, block, 0, s,
-                       in, out, chunk_vecs, bpr);
-  else
-    hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, false, false>), grid, block, 0, s,
-                       in, out, chunk_vecs, bpr);
-  return hipGetLastError();
+static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
+                                     const PtrTable &in, const PtrTable &out, size_t chunk_bytes) {
+  const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
+  const size_t seg_max = segment_of(t);
+  for (size_t off = 0; off < chunk_bytes; off += seg_max) {
+    const size_t seg = chunk_bytes - off < seg_max ? chunk_bytes - off : seg_max;
+    const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
+    const dim3 grid(bpr * N), block(t.block);
+    hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
+      hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value,
+                                             decltype(st_aux)::value>),
+                         grid, block, 0, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+      return hipGetLastError();
+    });
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 template <int N, int ORDER, int DT, typename V>
 static hipError_t launch_ar_unroll(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
-                                   const PtrTable &in, const PtrTable &out, size_t chunk_vecs) {
-  const int unroll = (N >= 16) ? 1 : (t.unroll >= 4 && N <= 8 ? 4 : (t.unroll >= 2 ? 2 : 1));
-  const uint32_t bpr = blocks_per_rank_for(dev, t, N, chunk_vecs, unroll);
-  const dim3 grid(bpr * N), block(t.block);
-  switch (unroll) {
-    case 4:
-      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, DT, V, 4>(s, grid, block, t, in, out, chunk_vecs, bpr);
-      [[fallthrough]];
-    case 2:
-      if constexpr (N <= 8) return launch_ar_nt<N, ORDER, DT, V, 2>(s, grid, block, t, in, out, chunk_vecs, bpr);
-      [[fallthrough]];
-    default:
-      return launch_ar_nt<N, ORDER, DT, V, 1>(s, grid, block, t, in, out, chunk_vecs, bpr);
+                                   const PtrTable &in, const PtrTable &out, size_t chunk_bytes) {
+  // 16 ranks already keep 16 loads per lane in flight; the bfloat16 add needs
+  // binary32 temporaries, which leaves no room for four vectors per rank.
+  const int unroll = (N >= 16) ? 1 : (t.unroll >= 4 ? 4 : (t.unroll >= 2 ? 2 : 1));
+  if constexpr (N <= 8) {
+    if constexpr (DT == DT_F16)
+      if (unroll == 4) return launch_ar_segments<N, ORDER, DT, V, 4>(s, dev, t, in, out, chunk_bytes);
+    if (unroll >= 2) return launch_ar_segments<N, ORDER, DT, V, 2>(s, dev, t, in, out, chunk_bytes);
   }
+  return launch_ar_segments<N, ORDER, DT, V, 1>(s, dev, t, in, out, chunk_bytes);
 }
-
 template <int N, int ORDER>
 static hipError_t launch_ar_vec(hipStream_t s, const DeviceInfo &dev, const Tuning &t, DType dtype,
                                 const PtrTable &in, const PtrTable &out, size_t chunk_elems,
                                 int vec_halves) {
+  const size_t bytes = chunk_elems * 2;
   if (dtype == DT_BF16) {
-    if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_BF16, h8>(s, dev, t, in, out, chunk_elems / 8);
-    return launch_ar_unroll<N, ORDER, DT_BF16, h4>(s, dev, t, in, out, chunk_elems / 4);
+    if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_BF16, h8>(s, dev, t, in, out, bytes);
+    return launch_ar_unroll<N, ORDER, DT_BF16, h4>(s, dev, t, in, out, bytes);
   }
-  if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_F16, h8>(s, dev, t, in, out, chunk_elems / 8);
-  return launch_ar_unroll<N, ORDER, DT_F16, h4>(s, dev, t, in, out, chunk_elems / 4);
+  if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_F16, h8>(s, dev, t, in, out, bytes);
+  return launch_ar_unroll<N, ORDER, DT_F16, h4>(s, dev, t, in, out, bytes);
 }
 
 hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
                                    Order order, DType dtype, const PtrTable &in, const PtrTable &out,
                                    size_t chunk_elems, int vec_halves) {
   if (chunk_elems == 0) return hipSuccess;
+  if (t.block < 64 || t.block > 1024 || t.block % 64) return hipErrorInvalidValue;
 #define VR_CASE(NN)                                                                              \
   case NN:                                                                                       \
     if (order == ORDER_BISECT) {                                                                 \
@@ -318,34 +331,41 @@ hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const T
 #undef VR_CASE
 }
 
+template <int N, typename V, int UNROLL>
+static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
+                                     const PtrTable &in, const PtrTable &out, size_t slice_bytes) {
+  const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
+  const size_t seg_max = segment_of(t);
+  for (size_t off = 0; off < slice_bytes; off += seg_max) {
+    const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
+    const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
+    const dim3 grid(bpr * N), block(t.block);
+    hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
+      hipLaunchKernelGGL((k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>),
+                         grid, block, 0, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+      return hipGetLastError();
+    });
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 template <int N, typename V>
 static hipError_t launch_ag(hipStream_t s, const DeviceInfo &dev, const Tuning &t, const PtrTable &in,
-                            const PtrTable &out, size_t slice_vecs) {
-  const int unroll = t.unroll >= 2 ? 2 : 1;
-  const uint32_t bpr = blocks_per_rank_for(dev, t, N, slice_vecs, unroll);
-  const dim3 grid(bpr * N), block(t.block);
-  if (unroll == 2) {
-    if (t.nt_store)
-      hipLaunchKernelGGL((k_direct_allgather<N, V, 2, true, true>), grid, block, 0, s, in, out, slice_vecs, bpr);
-    else
-      hipLaunchKernelGGL((k_direct_allgather<N, V, 2, false, false>), grid, block, 0, s, in, out, slice_vecs, bpr);
-  } else {
-    if (t.nt_store)
-      hipLaunchKernelGGL((k_direct_allgather<N, V, 1, true, true>), grid, block, 0, s, in, out, slice_vecs, bpr);
-    else
-      hipLaunchKernelGGL((k_direct_allgather<N, V, 1, false, false>), grid, block, 0, s, in, out, slice_vecs, bpr);
-  }
-  return hipGetLastError();
+                            const PtrTable &out, size_t slice_bytes) {
+  if (t.unroll >= 2) return launch_ag_segments<N, V, 2>(s, dev, t, in, out, slice_bytes);
+  return launch_ag_segments<N, V, 1>(s, dev, t, in, out, slice_bytes);
 }
 
 hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const Tuning &t, int nranks,
                                    const PtrTable &in, const PtrTable &out, size_t nelems,
                                    int vec_halves) {
   if (nelems == 0) return hipSuccess;
+  if (t.block < 64 || t.block > 1024 || t.block % 64) return hipErrorInvalidValue;
 #define VR_CASE(NN)                                                              \
   case NN:                                                                       \
-    if (vec_halves == 8) return launch_ag<NN, h8>(s, dev, t, in, out, nelems / 8); \
-    return launch_ag<NN, h4>(s, dev, t, in, out, nelems / 4);
+    if (vec_halves == 8) return launch_ag<NN, h8>(s, dev, t, in, out, nelems * 2); \
+    return launch_ag<NN, h4>(s, dev, t, in, out, nelems * 2);
   switch (nranks) {
     VR_CASE(2)
     VR_CASE(4)
@@ -357,39 +377,44 @@ hipError_t launch_direct_allgather(hipStream_t s, const DeviceInfo &dev, const T
 #undef VR_CASE
 }
 
+template <int MODE, int UNROLL>
+static hipError_t launch_probe_segments(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
+                                        char *dst, const char *src, size_t bytes) {
+  const size_t tile = (size_t)t.block * 16 * UNROLL;
+  const size_t seg_max = segment_of(t);
+  for (size_t off = 0; off < bytes; off += seg_max) {
+    const size_t seg = bytes - off < seg_max ? bytes - off : seg_max;
+    size_t blocks = (seg + tile - 1) / tile;
+    const size_t resident = (size_t)dev.cus * t.waves_per_cu / (t.block / 64);
+    if (!t.oneshot && blocks > resident) blocks = resident;
+    if (blocks == 0) blocks = 1;
+    const dim3 grid((uint32_t)blocks), block(t.block);
+    hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
+      hipLaunchKernelGGL((k_probe<MODE, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>), grid,
+                         block, 0, s, dst + off, src + off, (uint32_t)seg);
+      return hipGetLastError();
+    });
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 hipError_t launch_copy(hipStream_t s, const DeviceInfo &dev, const Tuning &t, void *dst,
                        const void *src, size_t bytes, int mode) {
-  const size_t vecs = bytes / 16;
-  if (vecs == 0) return hipSuccess;
-  const int unroll = t.unroll >= 4 ? 4 : 1;
-  const size_t tile = (size_t)t.block * unroll;
-  size_t blocks = (vecs + tile - 1) / tile;
-  const size_t resident = (size_t)dev.cus * t.waves_per_cu / (t.block / 64);
-  if (!t.oneshot && blocks > resident) blocks = resident;
-  const dim3 grid((uint32_t)blocks), block(t.block);
-  h8 *d = static_cast<h8 *>(dst);
-  const h8 *sp = static_cast<const h8 *>(src);
-#define VR_PROBE(M, U)                                                                    \
-  if (t.nt_load || t.nt_store)                                                            \
-    hipLaunchKernelGGL((k_probe<M, U, true>), grid, block, 0, s, d, sp, vecs);             \
-  else                                                                                    \
-    hipLaunchKernelGGL((k_probe<M, U, false>), grid, block, 0, s, d, sp, vecs);
-#define VR_PROBE_U(M)  \
-  if (unroll == 4) {   \
-    VR_PROBE(M, 4)     \
-  } else {             \
-    VR_PROBE(M, 1)     \
+  bytes -= bytes % 16;
+  if (bytes == 0) return hipSuccess;
+  if (t.block < 64 || t.block > 1024 || t.block % 64) return hipErrorInvalidValue;
+  char *d = static_cast<char *>(dst);
+  const char *sp = static_cast<const char *>(src);
+  const bool u4 = t.unroll >= 4;
+  switch (mode) {
+    case 1:
+      return u4 ? launch_probe_segments<1, 4>(s, dev, t, d, sp, bytes) : launch_probe_segments<1, 1>(s, dev, t, d, sp, bytes);
+    case 2:
+      return u4 ? launch_probe_segments<2, 4>(s, dev, t, d, sp, bytes) : launch_probe_segments<2, 1>(s, dev, t, d, sp, bytes);
+    default:
+      return u4 ? launch_probe_segments<0, 4>(s, dev, t, d, sp, bytes) : launch_probe_segments<0, 1>(s, dev, t, d, sp, bytes);
   }
-  if (mode == 1) {
-    VR_PROBE_U(1)
-  } else if (mode == 2) {
-    VR_PROBE_U(2)
-  } else {
-    VR_PROBE_U(0)
-  }
-#undef VR_PROBE_U
-#undef VR_PROBE
-  return hipGetLastError();
 }
 
 }  // namespace vr

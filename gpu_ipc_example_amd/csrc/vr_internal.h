@@ -29,8 +29,9 @@ struct Tuning {
   int block = 512;        // threads per work-group
   int waves_per_cu = 32;  // resident waves per CU the persistent grid asks for
   int unroll = 2;         // 16-byte vectors in flight per lane and rank
-  int nt_load = 1;
-  int nt_store = 1;
+  int nt_load = 1;         // 1: streaming loads (nt)
+  int nt_store = 1;        // 1: streaming stores (nt); 2: streaming and written through at agent scope (nt sc1)
+  size_t segment_bytes = 1ull << 30;  // bytes of a chunk one launch addresses (32-bit offsets); multiple of 16
   int oneshot = 0;        // 1: grid covers the whole buffer, no grid-stride loop
   uint32_t force_blocks_per_rank = 0;  // non-zero: use exactly this many blocks per rank
 };

@@ -293,6 +293,68 @@ def test_allgather_rejections(ctxs, oracle):
     assert e.value.code == "UNEVEN"
 
 
+def test_long_chunks_take_several_launches(ctxs, oracle):
+    """A launch addresses a chunk with 32-bit offsets; longer chunks are cut into
+    segments.  With the segment forced down to 4 KiB every size here takes several
+    launches per chunk, the last one a ragged piece."""
+    ctx = ctxs[8]
+    ctx.set_tuning(segment_kib=4)
+    try:
+        for algo, n in (("simple", 8 * 4 * 5000), ("bisect", 8 * 4 * 5000 + 32), ("small", 8 * 8 * 3333),
+                        ("simple_ring", 8 * 8 * 2048)):
+            ins = H.make_inputs(oracle, 8, n, 5150 + n)
+            want = H.expected(oracle, algo, ins)
+            got, _ = H.run_allreduce(ctx, algo, ins)
+            H.assert_all_ranks_equal(oracle, got, want, "%s n=%d segmented" % (algo, n))
+            got, _ = H.run_allreduce(ctx, algo, ins, inplace=False)
+            H.assert_all_ranks_equal(oracle, got, want, "%s n=%d segmented out-of-place" % (algo, n))
+        ins = H.make_inputs(oracle, 8, 8 * 1237, 99, DIST_UNIFORM, -2.0, 2.0)
+        want = oracle.allgather(ins)
+        for alias in (False, True):
+            got = run_allgather(ctx, "allgather_simple", ins, alias)
+            for r in range(8):
+                assert (got[r] == want).all(), (r, alias)
+    finally:
+        ctx.set_tuning(segment_kib=-1)
+
+
+@pytest.mark.parametrize("nt_store", [0, 1, 2])
+@pytest.mark.parametrize("nt_load", [0, 1])
+def test_every_cache_policy_gives_the_same_bits(ctxs, oracle, nt_load, nt_store):
+    ctx = ctxs[8]
+    ctx.set_tuning(nt_load=nt_load, nt_store=nt_store)
+    try:
+        for unroll in (1, 2, 4):
+            ctx.set_tuning(unroll=unroll)
+            n = 8 * 4 * 40001                               # ragged last tile at every unroll
+            ins = H.make_inputs(oracle, 8, n, 31 + unroll)
+            got, _ = H.run_allreduce(ctx, "bisect", ins)
+            H.assert_all_ranks_equal(oracle, got, oracle.bisect(ins), "unroll %d" % unroll)
+    finally:
+        ctx.set_tuning(nt_load=-1, nt_store=-1, unroll=-1)
+
+
+def test_nothing_is_written_past_the_end(ctxs, oracle):
+    """The last tile of a chunk hangs over its end; the hardware bounds check of the
+    buffer resource must drop those lanes (outputs carry 64 guard bytes here)."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    N, n = 8, 8 * 4 * 777
+    ins = H.make_inputs(oracle, N, n, 5)
+    src = H.RankBuffers(N, n)
+    src.upload(ins)
+    dst = [DeviceBuffer(n * 2 + 4096) for _ in range(N)]
+    for d in dst:
+        d.fill(0xAB)
+    ctxs[N].allreduce("simple", src.ptrs, n, outs=[d.ptr for d in dst])
+    ctxs[N].check()
+    want = oracle.rotated(ins)
+    for d in dst:
+        assert oracle.count_mismatch(d.download(np.uint16, n), want) == 0
+        assert (d.download(np.uint8, 4096, n * 2) == 0xAB).all()
+        d.free()
+    src.free()
+
+
 def test_work_groups_are_dealt_round_robin_over_the_xcds(ctxs):
     """The rank-to-XCD affinity the direct kernels are laid out for: consecutive
     work-groups of a launch go to consecutive XCDs (starting wherever the previous
