@@ -515,35 +515,46 @@ static bool ranges_partially_overlap(const void *a, const void *b, size_t bytes)
 
 // Launch heuristics of the direct kernels.  `read_bytes` / `write_bytes` are the
 // distinct bytes a launch reads and writes; what matters is how they compare with
-// the 256 MiB memory-side cache (Infinity Cache) in front of HBM.
+// the 256 MiB memory-side cache (Infinity Cache) in front of HBM.  Store policy 2
+// (streaming, written through at agent scope) is the fastest way to HBM but takes
+// the results out of the L2 a following in-place launch would read them from.
 static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes, size_t write_bytes,
                          bool in_place) {
   const size_t kMall = 256ull << 20;
   Tuning t;
   t.block = 256;
-  // The all-reduce keeps N loads per lane in flight and is DRAM-efficiency bound
-  // from 8 waves per CU on; the all-gather has one load per lane and needs the
-  // CU's full 32 waves to cover the latency.
-  t.waves_per_cu = a->allgather ? 32 : 8;
   t.unroll = 1;
-  if (a->latency_tuned) {
+  t.oneshot = 0;
+  if (a->allgather) {
+    // One load per lane: the CU's full 32 waves cover the latency.  Each input
+    // byte is read once (cached loads measured faster than streaming ones), each
+    // output byte is written once and not read back here.
+    t.waves_per_cu = 32;
+    t.nt_load = 0;
+    t.nt_store = 2;
+  } else if (a->latency_tuned) {
     // "small" family: every lane makes one trip; results stay cacheable for the
     // kernel that consumes them next.
+    t.waves_per_cu = 8;
     t.oneshot = 1;
     t.nt_load = 0;
     t.nt_store = 0;
   } else {
-    t.oneshot = 0;
     const size_t footprint = in_place ? read_bytes : read_bytes + write_bytes;
     if (footprint <= kMall) {            // everything can live in the memory-side cache
-      t.nt_load = 0;
-      t.nt_store = 0;
-    } else if (read_bytes <= kMall) {    // keep the inputs cacheable, stream the results past them
+      t.waves_per_cu = 8;
       t.nt_load = 0;
       t.nt_store = 1;
-    } else {                             // pure streaming
+    } else if (read_bytes <= kMall / 2) {  // inputs may still be resident; stream the results past them
+      t.waves_per_cu = 8;
+      t.nt_load = 0;
+      t.nt_store = 2;
+    } else {
+      // Pure streaming.  DRAM runs best with about 32 loads per CU in flight:
+      // N loads per lane times 4 waves (8 waves for two ranks).
+      t.waves_per_cu = ctx->nranks >= 4 ? 4 : 8;
       t.nt_load = 1;
-      t.nt_store = 1;
+      t.nt_store = 2;
     }
   }
   const TuningOverrides &o = ctx->tune;
@@ -843,7 +854,8 @@ static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, Tu
   d.block = 1024;
   d.waves_per_cu = 16;
   d.unroll = 4;
-  d.nt_load = d.nt_store = 1;
+  d.nt_load = 1;
+  d.nt_store = 2;
   d.oneshot = 0;
   const TuningOverrides &o = ctx->tune;
   if (o.block != -1) d.block = o.block;
