@@ -141,6 +141,10 @@ static int check_topology(const AlgoInfo *a, int nranks) {
 
 static inline size_t div_up(size_t x, size_t m) { return (x + m - 1) / m; }
 
+// Largest element count per rank: keeps nranks * nelems * 2 bytes (and the
+// all-gather's nranks times that) far inside size_t.
+static const size_t kMaxElems = (size_t)1 << 40;
+
 // calcWorkSize (allreduce.hpp:108-122): alignment is tested before divisibility.
 static int calc_work_size(uintptr_t addr, size_t bytes, size_t nchunks, size_t msg, size_t *work) {
   if (addr % msg != 0) return VR_ERR_UNALIGNED;
@@ -156,6 +160,7 @@ extern "C" int vr_check_allreduce(int algo, int nranks, const void *const bufs[]
   const AlgoInfo *a = algo_info(algo);
   if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
   if (!bufs) return fail(VR_ERR_INVALID, "null buffer table");
+  if (nelems > kMaxElems) return fail(VR_ERR_INVALID, "nelems too large");
   if (int rc = check_topology(a, nranks)) return rc;
   size_t work = 0;
   for (int r = 0; r < nranks; ++r) {
@@ -172,6 +177,7 @@ extern "C" int vr_check_allgather(int algo, int nranks, const void *const inputs
   const AlgoInfo *a = algo_info(algo);
   if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
   if (!inputs || !outputs) return fail(VR_ERR_INVALID, "null buffer table");
+  if (nelems > kMaxElems) return fail(VR_ERR_INVALID, "nelems too large");
   if (int rc = check_topology(a, nranks)) return rc;
   size_t work = 0;
   for (int r = 0; r < nranks; ++r) {
@@ -781,9 +787,15 @@ template <typename F>
 static int time_launches(hipStream_t s, int iters, float *ms_out, F &&launch) {
   if (iters <= 0 || !ms_out) return fail(VR_ERR_INVALID, "iters <= 0 or null ms_out");
   const int kBatch = 128;   // events in flight before the host waits
-  std::vector<hipEvent_t> ev(2 * (size_t)kBatch);
-  for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+  std::vector<hipEvent_t> ev(2 * (size_t)kBatch, nullptr);
   int rc = VR_OK;
+  for (auto &e : ev) {
+    hipError_t err = hipEventCreate(&e);
+    if (err != hipSuccess) {
+      rc = fail_hip(err, "hipEventCreate");
+      break;
+    }
+  }
   for (int done = 0; done < iters && rc == VR_OK; done += kBatch) {
     const int n = (iters - done < kBatch) ? iters - done : kBatch;
     for (int i = 0; i < n && rc == VR_OK; ++i) {
@@ -801,7 +813,8 @@ static int time_launches(hipStream_t s, int iters, float *ms_out, F &&launch) {
       ms_out[done + i] = ms;
     }
   }
-  for (auto &e : ev) (void)hipEventDestroy(e);
+  for (auto &e : ev)
+    if (e) (void)hipEventDestroy(e);
   return rc;
 }
 

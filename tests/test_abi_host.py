@@ -88,6 +88,12 @@ def test_topology_rules():
     assert vr.check_allreduce("bisect", 16, [0x1000] * 16, 64 * 16) == 128
 
 
+def test_absurd_sizes_are_rejected_before_any_arithmetic_overflows():
+    with pytest.raises(vr.VRError) as e:
+        vr.check_allreduce("small", 8, [0x1000] * 8, (1 << 62) + 32)
+    assert e.value.code == "INVALID"
+
+
 def test_launch_geometry_matches_getLaunchParam():
     # worked by hand from allreduce.hpp:37-62 with PVC constants
     assert vr.launch_geometry("simple", 2, 16384) == (5, 64, 1)       # 137 wires of 120 B, 32 per SS
