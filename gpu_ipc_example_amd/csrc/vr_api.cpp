@@ -218,7 +218,7 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
   int segment_kib = -1;
-  int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1;
+  int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1, wire_ahead = -1;
 };
 
 // Scratch of the wire transport: per virtual rank one scatter and one gather
@@ -249,6 +249,7 @@ struct vr_ctx {
 
 static const uint32_t kDefaultSpinLimit = 1u << 22;
 static const int kWireBlocksPerCu = 2;
+static const uint32_t kWireAhead = 4;
 
 static void wire_free(vr_ctx *c) {
   WireState &w = c->wire;
@@ -391,6 +392,7 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const uint64_t limit = c->spin_limit ? c->spin_limit : kDefaultSpinLimit;
   args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
   args.status = w.status;
+  args.ahead = c->tune.wire_ahead > 0 ? (uint32_t)c->tune.wire_ahead : kWireAhead;
   const bool cooperative = c->tune.wire_cooperative != 0;
   hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args,
                              cooperative, c->dtype);
@@ -464,6 +466,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
+  if (!strcmp(key, "wire_ahead")) return &ctx->tune.wire_ahead;
   return nullptr;
 }
 
@@ -485,6 +488,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
     if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))
       return fail(VR_ERR_INVALID, "segment_kib must be in [1, 1048576]");
+    if (!strcmp(key, "wire_ahead") && (value < 1 || value > kWireMaxSlots - 2))
+      return fail(VR_ERR_INVALID, "wire_ahead must be in [1,6]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
       if (value < 1 || value > 4) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be in [1,4]");
       if (ctx->wire.ready) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be set before the first wire-transport launch");

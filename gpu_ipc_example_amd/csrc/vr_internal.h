@@ -77,6 +77,7 @@ struct WireArgs {
   uint32_t waves_per_rank;   // wires each virtual rank runs (multiple of the flow's waves per column)
   uint32_t seq;              // first flag value of this launch
   uint32_t spin_limit;
+  uint32_t ahead;            // steps the scatters of the parallel flow run ahead of its gathers
   uint32_t *status;          // non-zero once any poll gave up
 };
 

@@ -361,21 +361,43 @@ static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, 
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
   constexpr int NSLOT = 8;
+  const uint32_t kAhead = a.ahead;   // 1 ... NSLOT - 2, checked by the host
   VR_WAVE_PROLOGUE;
   const Sinks<W, NSLOT> sk{a};
   const uint32_t y = wid % N, x_id = wid / N * N;
   const size_t columns = a.waves_per_rank / N;
   const char *src = static_cast<const char *>(a.in.p[r]) + y * chunk;
   char *dst = static_cast<char *>(a.out.p[r]) + y * chunk;
-  uint32_t t = 0;
-  for (size_t off = (size_t)(wid / N) * W::kWireBytes; off < chunk; off += columns * W::kWireBytes, ++t) {
-    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
-    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
-    typename W::Reg v = W::load(src + off, left, lane);
-    if ((int)y != r) {                               // scatter, then wait for the gather
-      W::send(sk.scat(y, x_id + r, s), sk.sflag(y, x_id + r, s), v, flag, lane);
+  const size_t first = (size_t)(wid / N) * W::kWireBytes, stride = columns * W::kWireBytes;
+  if ((int)y != r) {
+    // Scatter, then wait for the gather.  The scatters run kAhead steps ahead of
+    // the gathers waited for (kAhead + 1 of the ring's 8 slots in use; the
+    // reference's sub-groups stay within one step of each other,
+    // parallel_transmit.hpp:88-122), so the owner always finds its next messages
+    // waiting and the column runs at the owner's pace.
+    auto scatter = [&](size_t off, uint32_t step) {
+      const typename W::Reg p = W::load(src + off, bytes_left(chunk, off, W::kWireBytes), lane);
+      W::send(sk.scat(y, x_id + r, step % NSLOT), sk.sflag(y, x_id + r, step % NSLOT), p,
+              a.seq + step / NSLOT, lane);
+    };
+    for (uint32_t k = 0; k < kAhead; ++k)
+      if (first + k * stride < chunk) scatter(first + k * stride, k);
+    uint32_t t = 0;
+    for (size_t off = first; off < chunk; off += stride, ++t) {
+      const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+      const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+      if (off + kAhead * stride < chunk) scatter(off + kAhead * stride, t + kAhead);
+      typename W::Reg v;
       W::recv(sk.gath(r, x_id + y, s), sk.gflag(r, x_id + y, s), v, flag, lane, spin);
-    } else {                                         // wait, reduce, broadcast
+      W::store(dst + off, left, lane, v);
+    }
+  } else {
+    // Wait, reduce, broadcast.
+    uint32_t t = 0;
+    for (size_t off = first; off < chunk; off += stride, ++t) {
+      const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+      const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+      typename W::Reg v = W::load(src + off, left, lane);
       const char *ms[N - 1];
       const uint32_t *mf[N - 1];
       typename W::Reg m[N - 1];
@@ -392,8 +414,8 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
         const int next = (r + i + 1) % N;
         W::send(sk.gath(next, x_id + r, s), sk.gflag(next, x_id + r, s), v, flag, lane);
       }
+      W::store(dst + off, left, lane, v);
     }
-    W::store(dst + off, left, lane, v);
   }
 }
 
@@ -604,13 +626,19 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
   const char *src = static_cast<const char *>(a.in.p[r]);
   char *dst = static_cast<char *>(a.out.p[r]);
   uint32_t t = 0;
-  for (size_t off = (size_t)(wid / B) * W::kWireBytes; off < chunk; off += columns * W::kWireBytes, ++t) {
+  const size_t first = (size_t)(wid / B) * W::kWireBytes, stride = columns * W::kWireBytes;
+  // scatterFar runs one step ahead of the rest (two of the eight slots in use), so
+  // the pair sum of the next step never waits for the pair's load.
+  auto scatter_far = [&](size_t off, uint32_t step) {
+    const typename W::Reg f = W::load(src + far_off + off, bytes_left(chunk, off, W::kWireBytes), lane);
+    W::send(sk.scat(pair, far_base + wid, step % NSLOT), sk.sflag(pair, far_base + wid, step % NSLOT), f,
+            a.seq + step / NSLOT, lane);
+  };
+  if (first < chunk) scatter_far(first, 0);
+  for (size_t off = first; off < chunk; off += stride, ++t) {
     const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
-    {                                                 // scatterFar
-      const typename W::Reg f = W::load(src + far_off + off, left, lane);
-      W::send(sk.scat(pair, far_base + wid, s), sk.sflag(pair, far_base + wid, s), f, flag, lane);
-    }
+    if (off + stride < chunk) scatter_far(off + stride, t + 1);
     typename W::Reg v = W::load(src + close_off + off, left, lane);
     {                                                 // pair sum
       typename W::Reg m;

@@ -177,7 +177,8 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * for the wire transport "wire_fenced" (1 = the Rt64_128 family sends payload
  * lines with a separate flag word ordered by agent-scope release/acquire fences
  * instead of 64-byte segments with an embedded flag) and
- * "wire_cooperative" (0 = plain launch instead of a cooperative one), and
+ * "wire_cooperative" (0 = plain launch instead of a cooperative one),
+ * "wire_ahead" (1..6 steps the parallel flow's scatters run ahead of its gathers) and
  * "wire_blocks_per_cu" (1..4 resident work-groups per CU; set it before the first
  * wire-transport launch, it sizes the scratch).
  * -1 restores the library's own choice. */

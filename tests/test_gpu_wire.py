@@ -250,6 +250,24 @@ def test_plain_launch_instead_of_cooperative(oracle):
     ctx.close()
 
 
+@pytest.mark.parametrize("ahead", [1, 2, 6])
+def test_parallel_flow_scatters_running_ahead(oracle, ahead):
+    """The parallel flow's senders scatter up to `wire_ahead` steps before they wait
+    for a gather; with few wires per rank (a small user grid) every column takes
+    dozens of steps and wraps the 8-slot ring many times."""
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_ahead=ahead)
+    n = 8 * 4 * 30011
+    ins = H.make_inputs(oracle, 8, n, 6200 + ahead)
+    want = oracle.rotated(ins)
+    for algo in ("small", "parallel"):
+        for grid in (None, (1, 8, 16), (3, 8, 16)):
+            for inplace in (True, False):
+                got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, grid=grid, inplace=inplace)
+                H.assert_all_ranks_equal(oracle, got, want, "%s grid=%s inplace=%s" % (algo, grid, inplace))
+    ctx.close()
+
+
 def test_simple_transmit_ring_sections_wrap(ctxs, oracle):
     """Enough messages per sender to run through the 2 MiB ring sections several
     times in one launch (flag = seqNo + wraps), with small and large grids."""
