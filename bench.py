@@ -32,19 +32,26 @@ MEASURED_TRAFFIC_BYTES = {
     "cfg4": 167799218,
 }
 
+# Element type of the run (--dtype): 0 = binary16, 1 = bfloat16.  Buffers are
+# 2-byte elements either way; only the adds and the generated bit patterns differ.
+DTYPE = 0
+DTYPE_NAMES = {0: "f16", 1: "bf16"}
+
 WORKLOADS = {
     # name: (nranks, algo, nelems per rank, dist, p0, p1, seed)
     "cfg2": (8, "small", 524288, 1, 0.0, 1.0, 2000),
     "cfg3": (8, "bisect", 16777216, 1, 0.0, 0.02, 3000),
     "cfg4": (4, "allgather_simple", 4194304, 0, -2.0, 2.0, 4000),
+    # the 16-rank instantiation of bisect (allreduce.cpp:1020), same 256 MiB of inputs as cfg3
+    "bisect16": (16, "bisect", 8388608, 1, 0.0, 0.02, 6000),
 }
 
 
 def describe(name):
     n, algo, ne, dist, p0, p1, _ = WORKLOADS[name]
     d = ("N(%g,%g)" % (p0, p1)) if dist == 1 else ("U[%g,%g)" % (p0, p1))
-    return "%s: %d virtual ranks, %s, %d binary16/rank (%.3g MiB), %s" % (
-        name, n, algo, ne, ne * 2 / 2**20, d)
+    return "%s: %d virtual ranks, %s, %d %s/rank (%.3g MiB), %s" % (
+        name, n, algo, ne, "bfloat16" if DTYPE else "binary16", ne * 2 / 2**20, d)
 
 
 def algorithmic_bytes(name):
@@ -61,7 +68,8 @@ def setup(vr, binding, name, inplace, nsets=1):
     memory-side cache, so that every step really streams from and to HBM."""
     n, algo, ne, dist, p0, p1, seed = WORKLOADS[name]
     ctx = vr.VirtualRanks(n)
-    host = [binding.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
+    ctx.set_dtype(DTYPE)
+    host = [binding.generate(ne, seed + r, dist, p0, p1, dtype=DTYPE) for r in range(n)]
     sets = []
     for _ in range(nsets):
         ins = [binding.DeviceBuffer(ne * 2) for _ in range(n)]
@@ -140,16 +148,17 @@ def cpu_leg(name, gpu_results, budget_s):
 
     def reference(wname):
         n, algo, ne, dist, p0, p1, seed = WORKLOADS[wname]
-        host = [o.generate(ne, seed + r, dist, p0, p1) for r in range(n)]
-        fn = (o.allgather if algo.startswith("allgather")
-              else (o.bisect if algo == "bisect" else o.rotated))
-        return host, fn
+        host = [o.generate_dt(DTYPE, ne, seed + r, dist, p0, p1) for r in range(n)]
+        if algo.startswith("allgather"):
+            return host, o.allgather
+        mode = oracle_lib.ORDER_BISECT if algo == "bisect" else oracle_lib.ORDER_ROTATED
+        return host, (lambda ins: o.order_dt(DTYPE, mode, ins))
 
     mismatches = {}
     for wname, outs in gpu_results.items():
         host, fn = reference(wname)
         want = fn(host)
-        mismatches[wname] = int(sum(o.count_mismatch(g, want) for g in outs))
+        mismatches[wname] = int(sum(o.count_mismatch_dt(DTYPE, g, want) for g in outs))
 
     host, fn = reference(name)
     timing = {}
@@ -185,8 +194,9 @@ def sweep(vr, binding, args):
     size for each protocol, and the sizes at which the fastest protocol changes."""
     n = 8
     ctx = vr.VirtualRanks(n)
+    ctx.set_dtype(DTYPE)
     max_bytes = 256 << 20
-    host = binding.generate(max_bytes // 2, 5000, 1, 0.0, 1.0)
+    host = binding.generate(max_bytes // 2, 5000, 1, 0.0, 1.0, dtype=DTYPE)
     bufs = [binding.DeviceBuffer(max_bytes) for _ in range(n)]
     protos = [("small", vr.TRANSPORT_DIRECT), ("simple", vr.TRANSPORT_DIRECT),
               ("bisect", vr.TRANSPORT_DIRECT), ("parallel", vr.TRANSPORT_WIRE)]
@@ -239,6 +249,8 @@ def main():
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["copy"],
                     help="'copy' runs only the plain streaming copy (512 MiB per launch), the "
                          "known-size kernel that hardware-counter readings are scaled by")
+    ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"],
+                    help="element type of the adds (the reference instantiates both)")
     ap.add_argument("--inplace", action="store_true",
                     help="reference semantics: results overwrite the inputs (values saturate "
                          "after a few steps; traffic is identical)")
@@ -265,6 +277,9 @@ def main():
 
     import gpu_ipc_example_amd as vr
     from gpu_ipc_example_amd import binding
+
+    global DTYPE
+    DTYPE = 1 if args.dtype == "bf16" else 0
 
     if args.sweep:
         sweep(vr, binding, args)
@@ -325,11 +340,12 @@ def main():
     achieved = B / (k_avg * 1e-3) / 1e9
 
     result = {
-        "metric": "allreduce_algorithmic_hbm_bandwidth_8vrank_fp16_32MiB_per_rank"
+        "metric": ("allreduce_algorithmic_hbm_bandwidth_8vrank_%s_32MiB_per_rank"
+                   % ("bf16" if DTYPE else "fp16"))
                   if name == "cfg3" else "algorithmic_hbm_bandwidth_" + name,
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": DTYPE_NAMES[DTYPE], "data": "synthetic",
         "config": {"workload": describe(name), "virtual_ranks": n, "protocol": algo,
                    "bytes_per_rank": ne * 2, "in_place": bool(args.inplace),
                    "algorithmic_bytes_per_step": B, "buffer_sets_rotated": len(sets),
