@@ -224,6 +224,21 @@ def test_config3_bisect_32mib(ctxs, oracle):
     assert oracle.count_mismatch(want, oracle.rotated(ins)) > 1000   # the tree really differs
 
 
+@pytest.mark.parametrize("algo,transport", [("bisect", vr.TRANSPORT_DIRECT), ("simple", vr.TRANSPORT_DIRECT),
+                                            ("small", vr.TRANSPORT_DIRECT), ("parallel", vr.TRANSPORT_WIRE)])
+def test_full_size_closed_form(ctxs, algo, transport):
+    """The reference's own fixture at the headline size, checked without the oracle:
+    rank r holds (i % 32) * (r + 1), so every order gives (i % 32) * N (N + 1) / 2
+    exactly (utils.hpp:15-19, allreduce.cpp:537-548)."""
+    n = 16777216
+    from gpu_ipc_example_amd import binding
+    ins = [binding.fill_pattern(r, n) for r in range(8)]
+    want = ((np.arange(n, dtype=np.int64) % 32) * 36).astype(np.float16).view(np.uint16)
+    got, _ = H.run_allreduce(ctxs[8], algo, ins, transport=transport)
+    for r in range(8):
+        assert np.array_equal(got[r], want), (algo, r)
+
+
 def test_config5_sweep_sizes(ctxs, oracle):
     """4 KiB ... 256 MiB per rank in powers of two; the largest sizes are checked
     on one protocol each to keep host memory and time bounded."""
