@@ -625,29 +625,42 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
   const size_t far_off = (h ? 0 : (size_t)B * chunk) + y * chunk;
   const char *src = static_cast<const char *>(a.in.p[r]);
   char *dst = static_cast<char *>(a.out.p[r]);
-  uint32_t t = 0;
   const size_t first = (size_t)(wid / B) * W::kWireBytes, stride = columns * W::kWireBytes;
-  // scatterFar runs one step ahead of the rest (two of the eight slots in use), so
-  // the pair sum of the next step never waits for the pair's load.
+  // The stages that only feed other waves run ahead of the ones that wait (the
+  // reference keeps every sub-group inside one step, bisect_transmit.hpp:347-424,
+  // and so uses one of its eight slots): scatterFar two steps ahead, the pair sum
+  // and the close scatter one step ahead.  Same messages, slots and flag values.
   auto scatter_far = [&](size_t off, uint32_t step) {
     const typename W::Reg f = W::load(src + far_off + off, bytes_left(chunk, off, W::kWireBytes), lane);
     W::send(sk.scat(pair, far_base + wid, step % NSLOT), sk.sflag(pair, far_base + wid, step % NSLOT), f,
             a.seq + step / NSLOT, lane);
   };
-  if (first < chunk) scatter_far(first, 0);
-  for (size_t off = first; off < chunk; off += stride, ++t) {
-    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
-    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
-    if (off + stride < chunk) scatter_far(off + stride, t + 1);
-    typename W::Reg v = W::load(src + close_off + off, left, lane);
-    {                                                 // pair sum
-      typename W::Reg m;
-      W::recv(sk.scat(r, far_base + wid, s), sk.sflag(r, far_base + wid, s), m, flag, lane, spin);
-      W::add(v, m);
-    }
+  // Pair sum of a step, sent on to the chunk's owner unless this wave is the owner.
+  auto pair_sum = [&](size_t off, uint32_t step) {
+    const uint32_t s = step % NSLOT, flag = a.seq + step / NSLOT;
+    typename W::Reg v = W::load(src + close_off + off, bytes_left(chunk, off, W::kWireBytes), lane);
+    typename W::Reg m;
+    W::recv(sk.scat(r, far_base + wid, s), sk.sflag(r, far_base + wid, s), m, flag, lane, spin);
+    W::add(v, m);
     if ((int)y != l) {
       const int owner = 2 * (int)y + h;
       W::send(sk.scat(owner, wg + l, s), sk.sflag(owner, wg + l, s), v, flag, lane);
+    }
+    return v;
+  };
+  if (first >= chunk) return;
+  scatter_far(first, 0);
+  if (first + stride < chunk) scatter_far(first + stride, 1);
+  typename W::Reg cur = pair_sum(first, 0);
+  uint32_t t = 0;
+  for (size_t off = first; off < chunk; off += stride, ++t) {
+    const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
+    const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    if (off + 2 * stride < chunk) scatter_far(off + 2 * stride, t + 2);
+    typename W::Reg nxt = cur;
+    if (off + stride < chunk) nxt = pair_sum(off + stride, t + 1);
+    typename W::Reg v = cur;
+    if ((int)y != l) {
       W::recv(sk.gath(r, wg + y, s), sk.gflag(r, wg + y, s), v, flag, lane, spin);
     } else {
       const char *ms[B - 1];
@@ -674,6 +687,7 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
       W::recv(sk.gath(r, far_base + wid, s), sk.gflag(r, far_base + wid, s), m, flag, lane, spin);
       W::store(dst + far_off + off, left, lane, m);
     }
+    cur = nxt;
   }
 }
 
