@@ -77,8 +77,9 @@ typedef enum vr_algo {
  *          One pass over HBM; no scratch, no flags.  Default for every algo
  *          except VR_ALGO_PARALLEL.
  *  WIRE  : the reference's stage structure — scatter into the owner's sink,
- *          reduce, gather into every peer's sink — through the context's scratch
- *          with agent-scope release/acquire flag words, one persistent kernel
+ *          reduce, gather into every peer's sink — through the context's scratch,
+ *          with a flag inside every message (or, on request, separate flag words
+ *          ordered by agent-scope release/acquire fences), one persistent kernel
  *          whose workgroups are partitioned between the virtual ranks.  This is
  *          the form that carries over to several GPUs.  Default for
  *          VR_ALGO_PARALLEL. */
@@ -102,9 +103,10 @@ typedef struct vr_ctx vr_ctx;
 
 /* ---- lifetime --------------------------------------------------------------- */
 
-/* Creates a context for `nranks` virtual ranks on HIP device `device`.  Allocates
- * (and zeroes once, main.cpp:251) the wire-transport scratch: per rank a scatter
- * and a gather region plus flag words.  nranks must be 2, 4, 8 or 16. */
+/* Creates a context for `nranks` virtual ranks on HIP device `device`.  The
+ * wire-transport scratch (per rank a scatter and a gather region plus flag words)
+ * is allocated and zeroed once (main.cpp:241-251) by the first wire-transport
+ * launch; the direct transport needs none.  nranks must be 2, 4, 8 or 16. */
 int vr_ctx_create(int device, int nranks, vr_ctx **out);
 int vr_ctx_destroy(vr_ctx *ctx);
 int vr_ctx_nranks(const vr_ctx *ctx);
