@@ -1,5 +1,6 @@
 """Randomised parity sweep: random world size, protocol, transport, element
-count, alignment and in/out-of-place choice, each checked bit for bit against
+count, alignment, in/out-of-place choice and launch knobs (cache policy, unroll,
+residency, segment length, scatter run-ahead), each checked bit for bit against
 the oracle.  Seeds are fixed, so a failure names a reproducible case."""
 import random
 
@@ -32,10 +33,14 @@ def test_random_cases(oracle, seed):
         grid = None
         if rng.random() < 0.4:
             grid = (rng.choice((1, 2, 3, 7, 16, 33, 64)), rng.choice((4, 8, 12, 32, 64)), rng.choice((16, 32)))
+        knobs = dict(nt_load=rng.choice((-1, 0, 1)), nt_store=rng.choice((-1, 0, 1, 2)),
+                     unroll=rng.choice((-1, 1, 2, 4)), segment_kib=rng.choice((-1, -1, 4, 64)),
+                     waves_per_cu=rng.choice((-1, 1, 4, 32)), wire_ahead=rng.choice((-1, 1, 3, 6)))
+        ctxs[nranks].set_tuning(**knobs)
         ins = H.make_inputs(oracle, nranks, n, 10_000 * seed + 37 * case,
                             p1=rng.choice((0.02, 1.0, 30.0, 3000.0)))
-        what = "seed=%d case=%d %s N=%d n=%d transport=%d inplace=%s offset=%d grid=%s" % (
-            seed, case, algo, nranks, n, transport, inplace, offset, grid)
+        what = "seed=%d case=%d %s N=%d n=%d transport=%d inplace=%s offset=%d grid=%s knobs=%s" % (
+            seed, case, algo, nranks, n, transport, inplace, offset, grid, knobs)
         print(what, flush=True)
         got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=inplace, transport=transport,
                                     offset_bytes=offset, grid=grid)
