@@ -79,9 +79,11 @@ struct AlgoInfo {
       default: return WIRE_PARALLEL;
     }
   }
-  // Rt64 family -> self-validating 8-byte messages; Rt64_128 family -> 64-byte
-  // segments of 15 payload dwords and a flag.
-  WireFormat wire_format() const { return latency_tuned ? WIRE_FMT_LL : WIRE_FMT_LL64; }
+  // Rt64 -> self-validating 8-byte messages; Rt64_PCIE -> 16-byte messages with
+  // the flag twice; Rt64_128 family -> 64-byte segments of 15 payload dwords and a flag.
+  WireFormat wire_format() const {
+    return !latency_tuned ? WIRE_FMT_LL64 : msg_bytes == 16 ? WIRE_FMT_LL16 : WIRE_FMT_LL;
+  }
 };
 
 // message_t / wireCapacity: rt64.hpp:335-340 (8 B, 64 B), rt64_128.hpp:539-551 (8 B, 120 B),
@@ -218,7 +220,7 @@ extern "C" int vr_launch_geometry(int algo, int nranks, size_t nelems, vr_geomet
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
   int segment_kib = -1;
-  int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1, wire_ahead = -1;
+  int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1, wire_ahead = -1, wire_msg16 = -1;
 };
 
 // Scratch of the wire transport: per virtual rank one scatter and one gather
@@ -345,6 +347,7 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const WireFlow flow = a->wire_flow();
   WireFormat fmt = a->wire_format();
   if (fmt == WIRE_FMT_LL64 && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
+  if (fmt == WIRE_FMT_LL16 && c->tune.wire_msg16 == 0) fmt = WIRE_FMT_LL;
   const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
   const uint32_t waves_per_block = w.block_threads / 64;
   const uint32_t wpr_limit = w.blocks_per_rank_max * waves_per_block / psg * psg;
@@ -467,6 +470,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
   if (!strcmp(key, "wire_ahead")) return &ctx->tune.wire_ahead;
+  if (!strcmp(key, "wire_msg16")) return &ctx->tune.wire_msg16;
   return nullptr;
 }
 
@@ -480,7 +484,7 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
     if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
       return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
-    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") ||
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") || !strcmp(key, "wire_msg16") ||
          !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");

@@ -66,6 +66,7 @@ enum WireFormat : int {
   WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
   WIRE_FMT_LL64 = 1,  // 60 B payload + 4 B flag per 64-byte segment (Rt64_128 family)
   WIRE_FMT_FLAG = 2,  // 16 B payload lines + one fenced flag word per message
+  WIRE_FMT_LL16 = 3,  // 8 B payload + the flag twice per 16-byte store (Rt64_PCIE family)
 };
 constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
 

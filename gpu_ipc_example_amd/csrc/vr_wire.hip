@@ -9,12 +9,14 @@
 // 57-81,112-206 (Sequential), 262-278,333-516 (Ring), simple_transmit.hpp:16-179
 // and bisect_transmit.hpp:286-424,432-481, re-tiled for 64-lane wavefronts.
 //
-// Three wire formats:
-//   WireLL    (Rt64 family, rt64.hpp:334-341): every 8-byte store carries 4 bytes
+// Four wire formats:
+//   WireLL    (Rt64, rt64.hpp:334-341): every 8-byte store carries 4 bytes
 //             of payload and the 4-byte flag, so a message validates itself; the
 //             receiver re-polls until a wave-wide vote says every lane's flag is
 //             the expected one (the sub-group vote of parallel_transmit.hpp:95-101).
 //             Needs nothing but 8-byte store atomicity.
+//   WireLL16  (Rt64_PCIE, rt64.hpp:3-20): 16-byte stores of 8 bytes of payload and
+//             the flag twice.
 //   WireLL64  (Rt64_128 family): 15 payload dwords + 1 flag per 64-byte segment.
 //   WireFlag  (assumption-free alternative for the Rt64_128 family): payload lines
 //             plus a separate flag word, ordered by agent-scope release/acquire
@@ -132,6 +134,113 @@ struct WireLL {
           v[i].d[u] = (uint32_t)msg;
           ok = ok && (uint32_t)(msg >> 32) == flag;
         }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
+};
+
+// Rt64_PCIE (rt64.hpp:3-20, 100-134, 290-315): a lane's message is one 16-byte
+// store [d0, d1, flag, flag]: 8 bytes of payload, the flag twice.  The receiver
+// accepts a message once both flag words carry the expected value.  Only the
+// upper 8 bytes validate themselves, so like the reference's format this rests on
+// a lane's 16-byte store becoming visible as a whole (it lies inside one 64-byte
+// segment; the 64-byte format below rests on the stronger form of the same
+// property).  Moved with buffer instructions: 128-bit accesses with an
+// agent-scope policy, which the 64-bit atomic builtins cannot express.
+template <int U, int DT>
+struct WireLL16 {
+  static constexpr uint32_t kWireBytes = 64u * 8u * U;    // payload one wave moves per step
+  static constexpr uint32_t kSlotBytes = 64u * 16u * U;   // message bytes in the sink
+  static constexpr int kAuxAgent = 16;                             // sc1
+  static constexpr int kAuxAgentVolatile = (int)0x80000010u;       // sc1, never hoisted or merged
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  struct Reg {
+    uint32_t d[U][2];
+  };
+  // A slot address is the same in every lane of a wave (it depends on the wave's
+  // index only); saying so keeps the resource in scalar registers.
+  static __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const char *slot) {
+    const uint64_t a = reinterpret_cast<uint64_t>(slot);
+    // (the builtin returns int: go through uint32_t, or a low half with bit 31 set
+    // would sign-extend into the high half)
+    const uint64_t u = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                       ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char *>(u), 0, (int)kSlotBytes, 0x00020000);
+  }
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+    Reg r;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * 8u;
+      const uint2 z = off < left ? *reinterpret_cast<const uint2 *>(p + off) : make_uint2(0u, 0u);
+      r.d[u][0] = z.x;
+      r.d[u][1] = z.y;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t off = (u * 64u + lane) * 8u;
+      if (off < left) *reinterpret_cast<uint2 *>(p + off) = make_uint2(r.d[u][0], r.d[u][1]);
+    }
+  }
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64.hpp:126-134
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const h2 s = vadd<DT>(__builtin_bit_cast(h2, m.d[u][k]), __builtin_bit_cast(h2, v.d[u][k]));
+        v.d[u][k] = __builtin_bit_cast(uint32_t, s);
+      }
+  }
+  static __device__ __forceinline__ void send(char *slot, uint32_t *, const Reg &v, uint32_t flag,
+                                              uint32_t lane) {
+    const __amdgpu_buffer_rsrc_t rs = rsrc(slot);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const u32x4 msg = {v.d[u][0], v.d[u][1], flag, flag};
+      __builtin_amdgcn_raw_buffer_store_b128(msg, rs, (u * 64u + lane) * 16u, 0, kAuxAgent);
+    }
+  }
+  static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
+                                              uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    const __amdgpu_buffer_rsrc_t rs = rsrc(slot);
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const u32x4 msg = __builtin_amdgcn_raw_buffer_load_b128(rs, (u * 64u + lane) * 16u, 0, kAuxAgentVolatile);
+        v.d[u][0] = msg.x;
+        v.d[u][1] = msg.y;
+        ok = ok && msg.z == flag && msg.w == flag;
+      }
+      if (__all(ok)) return true;
+      if (spin.give_up(polls)) return false;
+    }
+  }
+  template <int M>
+  static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
+                                                   const uint32_t *const (&)[M], Reg (&v)[M],
+                                                   uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        const __amdgpu_buffer_rsrc_t rs = rsrc(slot[i]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const u32x4 msg = __builtin_amdgcn_raw_buffer_load_b128(rs, (u * 64u + lane) * 16u, 0, kAuxAgentVolatile);
+          v[i].d[u][0] = msg.x;
+          v[i].d[u][1] = msg.y;
+          ok = ok && msg.z == flag && msg.w == flag;
+        }
+      }
       if (__all(ok)) return true;
       if (spin.give_up(polls)) return false;
     }
@@ -701,6 +810,7 @@ __global__ void k_wire_clear(uint64_t *p, size_t n64) {
 
 // Messages per lane and step for each format; every slot stays within 2 KiB.
 constexpr int kUnrollLL = 4;     // 1 KiB payload in a 2 KiB message
+constexpr int kUnrollLL16 = 2;   // 1 KiB payload in a 2 KiB message
 constexpr int kUnrollLL64 = 4;   // 1920 B payload in a 2 KiB message
 constexpr int kUnrollFlag = 2;   // 2 KiB payload (16-byte lanes), flag word elsewhere
 
@@ -745,6 +855,7 @@ uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   switch (fmt) {
     case WIRE_FMT_LL: return WireLL<kUnrollLL, DT_F16>::kWireBytes;
     case WIRE_FMT_LL64: return WireLL64<kUnrollLL64, DT_F16>::kWireBytes;
+    case WIRE_FMT_LL16: return WireLL16<kUnrollLL16, DT_F16>::kWireBytes;
     default:
       return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16>::kWireBytes
                              : WireFlag<kUnrollFlag, h4, DT_F16>::kWireBytes;
@@ -760,6 +871,8 @@ static hipError_t launch_wire_dt(hipStream_t s, WireFlow flow, WireFormat fmt, i
     return launch_flow<WireLL<kUnrollLL, DT>>(s, flow, nranks, grid, block, args, cooperative);
   if (fmt == WIRE_FMT_LL64)
     return launch_flow<WireLL64<kUnrollLL64, DT>>(s, flow, nranks, grid, block, args, cooperative);
+  if (fmt == WIRE_FMT_LL16)
+    return launch_flow<WireLL16<kUnrollLL16, DT>>(s, flow, nranks, grid, block, args, cooperative);
   if (vec_halves == 8)
     return launch_flow<WireFlag<kUnrollFlag, h8, DT>>(s, flow, nranks, grid, block, args, cooperative);
   return launch_flow<WireFlag<kUnrollFlag, h4, DT>>(s, flow, nranks, grid, block, args, cooperative);

@@ -180,7 +180,9 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * lines with a separate flag word ordered by agent-scope release/acquire fences
  * instead of 64-byte segments with an embedded flag) and
  * "wire_cooperative" (0 = plain launch instead of a cooperative one),
- * "wire_ahead" (1..6 steps the parallel flow's scatters run ahead of its gathers) and
+ * "wire_ahead" (1..6 steps the parallel flow's scatters run ahead of its gathers),
+ * "wire_msg16" (0 = the Rt64_PCIE family sends self-validating 8-byte messages
+ * instead of 16-byte stores that carry the flag twice) and
  * "wire_blocks_per_cu" (1..4 resident work-groups per CU; set it before the first
  * wire-transport launch, it sizes the scratch).
  * -1 restores the library's own choice. */

@@ -268,6 +268,22 @@ def test_parallel_flow_scatters_running_ahead(oracle, ahead):
     ctx.close()
 
 
+def test_sixteen_byte_messages_can_be_swapped_for_eight_byte_ones(oracle):
+    """The Rt64_PCIE family sends [d0, d1, flag, flag] in one 16-byte store; with
+    wire_msg16=0 it falls back to self-validating 8-byte messages.  Same bits."""
+    ctx = vr.VirtualRanks(8)
+    n = 8 * 8 * 4099
+    ins = H.make_inputs(oracle, 8, n, 6400)
+    want = oracle.rotated(ins)
+    for msg16 in (1, 0, -1):
+        ctx.set_tuning(wire_msg16=msg16)
+        for algo in ("small_pcie_p", "small_ring", "small_pcie"):
+            for inplace in (True, False):
+                got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, inplace=inplace)
+                H.assert_all_ranks_equal(oracle, got, want, "%s msg16=%d" % (algo, msg16))
+    ctx.close()
+
+
 def test_simple_transmit_ring_sections_wrap(ctxs, oracle):
     """Enough messages per sender to run through the 2 MiB ring sections several
     times in one launch (flag = seqNo + wraps), with small and large grids."""
@@ -281,10 +297,12 @@ def test_simple_transmit_ring_sections_wrap(ctxs, oracle):
             assert oracle.count_mismatch(got[r], got[0]) == 0, (grid, r)
 
 
-@pytest.mark.parametrize("algo", ["simple", "bisect", "simple_ring", "small", "simple_transmit"])
+@pytest.mark.parametrize("algo", ["simple", "bisect", "simple_ring", "small", "simple_transmit",
+                                  "small_ring", "small_pcie"])
 def test_embedded_flag_formats_under_repetition(ctxs, oracle, algo):
-    """Many launches over the same sinks: every 64-byte segment (Rt64_128 family)
-    and every 8-byte message (Rt64 family) must arrive whole every time."""
+    """Many launches over the same sinks: every 64-byte segment (Rt64_128 family),
+    every 8-byte message (Rt64) and every 16-byte message (Rt64_PCIE) must arrive
+    whole every time."""
     from gpu_ipc_example_amd.binding import DeviceBuffer
     ctx = ctxs[8]
     n = 8 * 8192
