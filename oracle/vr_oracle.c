@@ -443,10 +443,25 @@ typedef struct {
   int wire;      /* VRO_WIRE_*                                   */
 } wire_fmt;
 
+/* Payload dwords per wire and the per-lane load shape (lanes that load x dwords each):
+ * Rt64 16 x 1 (rt64.hpp:339,566-583), Rt64_128 15 x 2 (rt64_128.hpp:551,563-583),
+ * Rt64_PCIE 16 x 2 (rt64.hpp:8,26-31), Rt64_128_PCIE 15 x 4 (rt64_128.hpp:14-21,33-52). */
+enum { MAX_DW = 64 };
+static int fmt_lanes(int wire) { return (wire == VRO_WIRE_RT64 || wire == VRO_WIRE_RT64_PCIE) ? 16 : 15; }
+static int fmt_dw_per_lane(int wire) {
+  switch (wire) {
+    case VRO_WIRE_RT64: return 1;
+    case VRO_WIRE_RT64_128: return 2;
+    case VRO_WIRE_RT64_PCIE: return 2;
+    default: return 4;
+  }
+}
+static int fmt_is_pcie(int wire) { return wire == VRO_WIRE_RT64_PCIE || wire == VRO_WIRE_RT64_128_PCIE; }
+
 static wire_fmt make_fmt(int wire) {
   wire_fmt f;
   f.wire = wire;
-  f.cap_dw = (wire == VRO_WIRE_RT64) ? 16 : 30;
+  f.cap_dw = fmt_lanes(wire) * fmt_dw_per_lane(wire);
   return f;
 }
 
@@ -485,9 +500,9 @@ static int unpack_msg(const wire_fmt *f, const uint32_t *msg, uint32_t *payload,
 
 /* Predicated load of one wire: lanes whose first element index is >= n_left stay 0. */
 static void load_wire(const wire_fmt *f, uint32_t *payload, const uint16_t *src, size_t n_left) {
-  const int lanes = (f->wire == VRO_WIRE_RT64) ? 16 : 15;
-  const int dw_per_lane = (f->wire == VRO_WIRE_RT64) ? 1 : 2;
-  memset(payload, 0, sizeof(uint32_t) * 32);
+  const int lanes = fmt_lanes(f->wire);
+  const int dw_per_lane = fmt_dw_per_lane(f->wire);
+  memset(payload, 0, sizeof(uint32_t) * MAX_DW);
   for (int l = 0; l < lanes; ++l) {
     const size_t off = (size_t)l * dw_per_lane * 2;       /* in halves */
     if (off < n_left) memcpy(payload + l * dw_per_lane, src + off, 4u * dw_per_lane);
@@ -495,8 +510,8 @@ static void load_wire(const wire_fmt *f, uint32_t *payload, const uint16_t *src,
 }
 
 static void store_wire(const wire_fmt *f, uint16_t *dst, const uint32_t *payload, size_t n_left) {
-  const int lanes = (f->wire == VRO_WIRE_RT64) ? 16 : 15;
-  const int dw_per_lane = (f->wire == VRO_WIRE_RT64) ? 1 : 2;
+  const int lanes = fmt_lanes(f->wire);
+  const int dw_per_lane = fmt_dw_per_lane(f->wire);
   for (int l = 0; l < lanes; ++l) {
     const size_t off = (size_t)l * dw_per_lane * 2;
     if (off < n_left) memcpy(dst + off, payload + l * dw_per_lane, 4u * dw_per_lane);
@@ -522,7 +537,7 @@ static void accum(uint32_t *v, const uint32_t *m, int ndw) {
 int vro_emulate_parallel(uint16_t *const io[], int nranks, size_t n, int wire_kind, int groups,
                          int subgroups, uint32_t seq_no) {
   const int N = nranks;
-  if (N < 2 || N > MAXR || n % (size_t)N) return -2;
+  if (N < 2 || N > MAXR || n % (size_t)N || fmt_is_pcie(wire_kind)) return -2;
   const wire_fmt f = make_fmt(wire_kind);
   const size_t W = (size_t)groups * (size_t)subgroups;       /* sub-groups in the launch */
   if (W < (size_t)N || W % (size_t)N || W > MAXLAUNCH) return -3;  /* reference would spin / overrun */
@@ -540,7 +555,7 @@ int vro_emulate_parallel(uint16_t *const io[], int nranks, size_t n, int wire_ki
     scat[r] = calloc(buf_dw, 4);
     gath[r] = calloc(buf_dw, 4);
   }
-  uint32_t(*regs)[32] = malloc(sizeof(uint32_t[32]) * (size_t)N * (size_t)N);
+  uint32_t(*regs)[MAX_DW] = malloc(sizeof(uint32_t[MAX_DW]) * (size_t)N * (size_t)N);
   int rc = 0;
 
   size_t t = 0;
@@ -552,7 +567,7 @@ int vro_emulate_parallel(uint16_t *const io[], int nranks, size_t n, int wire_ki
       if (wire_off >= work_bytes) continue;                   /* workLeft <= 0           */
       const size_t off_el = wire_off / 2, left = work_elems - off_el;
       const size_t x_id = x * (size_t)N;
-      uint32_t msg[32], tmp[32];
+      uint32_t msg[32], tmp[MAX_DW];
       /* Phase A: every rank's sub-group y loads chunk y; non-owners scatter. */
       for (int r = 0; r < N; ++r)
         for (int y = 0; y < N; ++y) {
@@ -614,7 +629,7 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire_kind, 
   enum { NSLOT = 4 };
   /* sinks: [rank][peer][slot][wire] of {32 payload dwords, flag} */
   typedef struct {
-    uint32_t p[32];
+    uint32_t p[MAX_DW];
     uint32_t flag;
   } cell;
   const size_t cells = (size_t)N * NSLOT * W;
@@ -633,7 +648,7 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire_kind, 
       const size_t wire_off = w * cap + goff;
       if (wire_off >= work_bytes) continue;
       const size_t off_el = wire_off / 2, left = work_elems - off_el;
-      uint32_t v[32];
+      uint32_t v[MAX_DW];
       /* step 0: rank r sends chunk r to r+1 */
       for (int r = 0; r < N; ++r) {
         const int peer = r, next = (r + 1) % N;
@@ -689,6 +704,146 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire_kind, 
   return rc;
 }
 
+
+/* SequentialTransmit::run (sequential_transmit.hpp:57-81, 83-207): one sub-group per
+ * wire does everything its rank owes the wire.  Sinks are indexed
+ * [sender's region][slot][wire] (the ringPtr typedef, l.54, indexed [tStep%nSlot][wireId]). */
+int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire_kind, int groups,
+                           int subgroups, uint32_t seq_no) {
+  const int N = nranks;
+  if (N < 2 || N > MAXR || n % (size_t)N) return -2;
+  const wire_fmt f = make_fmt(wire_kind);
+  const size_t W = (size_t)groups * (size_t)subgroups;       /* parallel_sg = 1          */
+  if (W == 0 || W > MAXLAUNCH) return -3;
+  const size_t work_elems = n / (size_t)N, work_bytes = work_elems * 2;
+  const size_t cap = (size_t)f.cap_dw * 4;
+  const size_t loop = W * cap;
+  enum { NSLOT = 4 };
+  typedef struct {
+    uint32_t p[MAX_DW];
+    uint32_t flag;
+  } cell;
+  const size_t cells = (size_t)N * NSLOT * W;
+  cell *scat[MAXR], *gath[MAXR];
+  for (int r = 0; r < N; ++r) {
+    scat[r] = calloc(cells, sizeof(cell));
+    gath[r] = calloc(cells, sizeof(cell));
+  }
+#define CELL(buf, region, slot, w) ((buf) + (((size_t)(region) * NSLOT + (slot)) * W + (w)))
+  int rc = 0;
+  size_t t = 0;
+  for (size_t goff = 0; goff < work_bytes && rc == 0; goff += loop, ++t) {
+    const uint32_t flag = seq_no + (uint32_t)(t / NSLOT);
+    const size_t slot = t % NSLOT;
+    for (size_t w = 0; w < W && rc == 0; ++w) {
+      const size_t wire_off = w * cap + goff;
+      if (wire_off >= work_bytes) continue;
+      const size_t off_el = wire_off / 2, left = work_elems - off_el;
+      /* scatter: rank r sends chunk `next` into next's sink, region r (l.96-117) */
+      for (int r = 0; r < N; ++r)
+        for (int i = 0; i < N - 1; ++i) {
+          const int next = (r + i + 1) % N;
+          cell *c = CELL(scat[next], r, slot, w);
+          load_wire(&f, c->p, io[r] + (size_t)next * work_elems + off_el, left);
+          c->flag = flag;
+        }
+      /* reduce own chunk with the peers' messages in order rank+1, rank+2, ... (l.130-171),
+       * gather-push (l.173-177), store (l.181-186) */
+      for (int r = 0; r < N && rc == 0; ++r) {
+        uint32_t v[MAX_DW];
+        load_wire(&f, v, io[r] + (size_t)r * work_elems + off_el, left);
+        for (int i = 0; i < N - 1; ++i) {
+          const int next = (r + i + 1) % N;
+          const cell *c = CELL(scat[r], next, slot, w);
+          if (c->flag != flag) { rc = -1; break; }
+          accum(v, c->p, f.cap_dw);
+        }
+        if (rc) break;
+        for (int i = 0; i < N - 1; ++i) {
+          const int next = (r + i + 1) % N;
+          cell *c = CELL(gath[next], r, slot, w);
+          memcpy(c->p, v, sizeof v);
+          c->flag = flag;
+        }
+        store_wire(&f, io[r] + (size_t)r * work_elems + off_el, v, left);
+      }
+      /* collect the other chunks (l.190-206) */
+      for (int r = 0; r < N && rc == 0; ++r)
+        for (int i = 0; i < N - 1; ++i) {
+          const int next = (r + i + 1) % N;
+          const cell *c = CELL(gath[r], next, slot, w);
+          if (c->flag != flag) { rc = -1; break; }
+          store_wire(&f, io[r] + (size_t)next * work_elems + off_el, c->p, left);
+        }
+    }
+  }
+  for (int r = 0; r < N; ++r) {
+    free(scat[r]);
+    free(gath[r]);
+  }
+  return rc;
+}
+
+/* AllGather<T,N,Proto,RingTransmit,16> (allgather.hpp:79-100 + sequential_transmit.hpp:
+ * 474-516, 396-428): the whole input is one work item list (workSize = bytes of one
+ * input); rank r stores its own slice, sends it on, forwards N-2 slices and stores the
+ * last.  out[r] holds N * n halves; out[r] + r * n may be in[r] itself (l.496-497). */
+int vro_emulate_allgather_ring(uint16_t *const out[], const uint16_t *const in[], int nranks, size_t n,
+                               int wire_kind, int groups, int subgroups, uint32_t seq_no) {
+  const int N = nranks;
+  if (N < 2 || N > MAXR || (N & (N - 1))) return -2;          /* uint32 wrap needs 2^k */
+  const wire_fmt f = make_fmt(wire_kind);
+  const size_t W = (size_t)groups * (size_t)subgroups;
+  if (W == 0 || W > MAXLAUNCH) return -3;
+  const size_t work_elems = n, work_bytes = n * 2;
+  const size_t cap = (size_t)f.cap_dw * 4;
+  const size_t loop = W * cap;
+  enum { NSLOT = 4 };
+  typedef struct {
+    uint32_t p[MAX_DW];
+    uint32_t flag;
+  } cell;
+  const size_t cells = (size_t)N * NSLOT * W;
+  cell *gath[MAXR];
+  for (int r = 0; r < N; ++r) gath[r] = calloc(cells, sizeof(cell));
+  int rc = 0;
+  size_t t = 0;
+  for (size_t goff = 0; goff < work_bytes && rc == 0; goff += loop, ++t) {
+    const uint32_t flag = seq_no + (uint32_t)(t / NSLOT);
+    const size_t slot = (seq_no + t) % NSLOT;
+    for (size_t w = 0; w < W && rc == 0; ++w) {
+      const size_t wire_off = w * cap + goff;
+      if (wire_off >= work_bytes) continue;
+      const size_t off_el = wire_off / 2, left = work_elems - off_el;
+      /* own slice: store unless the input already is the output slot, send on */
+      for (int r = 0; r < N; ++r) {
+        const int peer = r, next = (r + 1) % N;
+        cell *c = CELL(gath[next], peer, slot, w);
+        load_wire(&f, c->p, in[r] + off_el, left);
+        c->flag = flag;
+        uint16_t *o = out[r] + (size_t)peer * work_elems + off_el;
+        if (o != in[r] + off_el) store_wire(&f, o, c->p, left);
+      }
+      /* p_idx = -1, -2, ...: receive slice (rank - i), forward it except on the last hop */
+      for (int i = 1; i < N && rc == 0; ++i)
+        for (int r = 0; r < N; ++r) {
+          const int peer = (r + N - i) % N, next = (r + 1) % N;
+          const cell *c = CELL(gath[r], peer, slot, w);
+          if (c->flag != flag) { rc = -1; break; }
+          if (i < N - 1) {
+            cell *d = CELL(gath[next], peer, slot, w);
+            memcpy(d->p, c->p, sizeof c->p);
+            d->flag = flag;
+          }
+          store_wire(&f, out[r] + (size_t)peer * work_elems + off_el, c->p, left);
+        }
+    }
+  }
+#undef CELL
+  for (int r = 0; r < N; ++r) free(gath[r]);
+  return rc;
+}
+
 int vro_emulate_bisect(uint16_t *const io[], int nranks, size_t n, int groups, int subgroups,
                        uint32_t seq_no) {
   const int N = nranks, B = nranks / 2;
@@ -706,7 +861,7 @@ int vro_emulate_bisect(uint16_t *const io[], int nranks, size_t n, int groups, i
     scat[r] = calloc(buf_dw, 4);
     gath[r] = calloc(buf_dw, 4);
   }
-  uint32_t(*regs)[32] = malloc(sizeof(uint32_t[32]) * (size_t)N * (size_t)B);
+  uint32_t(*regs)[MAX_DW] = malloc(sizeof(uint32_t[MAX_DW]) * (size_t)N * (size_t)B);
   int rc = 0;
   size_t t = 0;
   /* Element offset of rank r's close / far half (bisect_transmit.hpp:439-444). */
@@ -720,7 +875,7 @@ int vro_emulate_bisect(uint16_t *const io[], int nranks, size_t n, int groups, i
       if (wire_off >= work_bytes) continue;
       const size_t off_el = wire_off / 2, left = work_elems - off_el;
       const size_t wg = x * (size_t)B;                        /* wireId_g                */
-      uint32_t msg[32], tmp[32];
+      uint32_t msg[32], tmp[MAX_DW];
       /* scatterFar: send the half this rank does not own to the pair rank. */
       for (int r = 0; r < N; ++r)
         for (int y = 0; y < B; ++y) {

@@ -110,6 +110,8 @@ size_t vro_count_mismatch(const uint16_t *a, const uint16_t *b, size_t n);
 enum {
   VRO_WIRE_RT64 = 0,      /* rt64.hpp:334-341      64 B payload / 128 B message (SG16) */
   VRO_WIRE_RT64_128 = 1,  /* rt64_128.hpp:538-553 120 B payload / 128 B message        */
+  VRO_WIRE_RT64_PCIE = 2,      /* rt64.hpp:3-9       128 B payload / 256 B message (ring, sequential, all-gather) */
+  VRO_WIRE_RT64_128_PCIE = 3,  /* rt64_128.hpp:3-21  240 B payload / 256 B message (ring, sequential, all-gather) */
 };
 
 /* AllReduce<T,N,Proto,ParallelTransmit,16>::operator() for every rank
@@ -121,6 +123,15 @@ int vro_emulate_parallel(uint16_t *const io[], int nranks, size_t n, int wire,
  * wire format does not change the arithmetic so only payload moves here. */
 int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire,
                      int groups, int subgroups, uint32_t seq_no);
+
+/* AllReduce<T,N,Proto,SequentialTransmit,16> (sequential_transmit.hpp:57-81, 83-207). */
+int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire,
+                           int groups, int subgroups, uint32_t seq_no);
+
+/* AllGather<T,N,Proto,RingTransmit,16> (allgather.hpp:79-100 + sequential_transmit.hpp:
+ * 474-516).  out[r] holds nranks * n halves; out[r] + r * n may alias in[r]. */
+int vro_emulate_allgather_ring(uint16_t *const out[], const uint16_t *const in[], int nranks, size_t n,
+                               int wire, int groups, int subgroups, uint32_t seq_no);
 
 /* bisectPAllReduce<T,N,BisectPTransmit,16> (allreduce.hpp:275-296 +
  * bisect_transmit.hpp:286-424). */

@@ -15,7 +15,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 SO = os.path.join(ORACLE_DIR, "libvr_oracle.so")
 
 DIST_UNIFORM, DIST_NORMAL = 0, 1
-WIRE_RT64, WIRE_RT64_128 = 0, 1
+WIRE_RT64, WIRE_RT64_128, WIRE_RT64_PCIE, WIRE_RT64_128_PCIE = 0, 1, 2, 3
 ORDER_RANK, ORDER_ROTATED, ORDER_BISECT = 0, 1, 2
 F16, BF16 = 0, 1
 
@@ -68,13 +68,16 @@ class Oracle:
         L.vro_allgather.argtypes = [_u16p, C.POINTER(_u16p), C.c_int, C.c_size_t]
         L.vro_count_mismatch.restype = C.c_size_t
         L.vro_count_mismatch.argtypes = [_u16p, _u16p, C.c_size_t]
-        for name in ("parallel", "ring"):
+        for name in ("parallel", "ring", "sequential"):
             f = getattr(L, "vro_emulate_" + name)
             f.restype = C.c_int
             f.argtypes = [C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_uint32]
         L.vro_emulate_bisect.restype = C.c_int
         L.vro_emulate_bisect.argtypes = [C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int, C.c_int,
                                          C.c_uint32]
+        L.vro_emulate_allgather_ring.restype = C.c_int
+        L.vro_emulate_allgather_ring.argtypes = [C.POINTER(_u16p), C.POINTER(_u16p), C.c_int, C.c_size_t,
+                                                 C.c_int, C.c_int, C.c_int, C.c_uint32]
         L.vro_bf16_add.restype = C.c_uint16
         L.vro_bf16_add.argtypes = [C.c_uint16, C.c_uint16]
         L.vro_f64_to_bf16.restype = C.c_uint16
@@ -204,6 +207,28 @@ class Oracle:
         rc = self.lib.vro_emulate_ring(_ptr_array(io), len(io), len(io[0]), wire, groups,
                                        subgroups, seq_no)
         return rc, io
+
+    def emulate_sequential(self, ins, wire, groups, subgroups, seq_no=1):
+        io = [a.copy() for a in ins]
+        rc = self.lib.vro_emulate_sequential(_ptr_array(io), len(io), len(io[0]), wire, groups,
+                                             subgroups, seq_no)
+        return rc, io
+
+    def emulate_allgather_ring(self, ins, wire, groups, subgroups, seq_no=1, alias_own_slot=False):
+        """Returns rc and the N output arrays (N * n halves each), pre-filled with 0x0101
+        like main.cpp:300 does.  alias_own_slot: rank r's input is slot r of its output."""
+        N, n = len(ins), len(ins[0])
+        outs = [np.full(N * n, 0x0101, np.uint16) for _ in range(N)]
+        srcs = []
+        for r in range(N):
+            if alias_own_slot:
+                outs[r][r * n:(r + 1) * n] = ins[r]
+                srcs.append(outs[r][r * n:(r + 1) * n])     # a view: same memory
+            else:
+                srcs.append(ins[r].copy())
+        rc = self.lib.vro_emulate_allgather_ring(_ptr_array(outs), _ptr_array(srcs), N, n, wire, groups,
+                                                 subgroups, seq_no)
+        return rc, outs
 
     def emulate_bisect(self, ins, groups, subgroups, seq_no=1):
         io = [a.copy() for a in ins]

@@ -13,7 +13,8 @@ Pins used (none of them re-types the oracle's own formula):
 import numpy as np
 import pytest
 
-from tests.oracle_lib import WIRE_RT64, WIRE_RT64_128, DIST_NORMAL, DIST_UNIFORM
+from tests.oracle_lib import (WIRE_RT64, WIRE_RT64_128, WIRE_RT64_PCIE, WIRE_RT64_128_PCIE, DIST_NORMAL,
+                              DIST_UNIFORM)
 
 
 def h(x):
@@ -209,6 +210,61 @@ def test_emulate_ring_matches_rotated(oracle, nranks, wire):
             assert rc == 0
             for r in range(nranks):
                 assert (io[r] == want).all(), (n, g, w, r)
+
+
+ALL_WIRES = [WIRE_RT64, WIRE_RT64_128, WIRE_RT64_PCIE, WIRE_RT64_128_PCIE]
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("wire", ALL_WIRES)
+def test_emulate_sequential_matches_rotated(oracle, nranks, wire):
+    """SequentialTransmit (sequential_transmit.hpp:83-207) moves other messages through
+    other sinks than ParallelTransmit but associates the same way."""
+    for n in (8 * nranks, 8 * nranks * 15, 16384, 8 * nranks * 1237):
+        ins = [oracle.generate(n, 41 + r, DIST_NORMAL, 0.0, 1.0) for r in range(nranks)]
+        want = oracle.rotated(ins)
+        for g, w in GEOMS[:6] + [(3, 4)]:
+            rc, io = oracle.emulate_sequential(ins, wire, g, w, seq_no=9)
+            assert rc == 0
+            for r in range(nranks):
+                assert (io[r] == want).all(), (n, g, w, r)
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("wire", [WIRE_RT64_PCIE, WIRE_RT64_128_PCIE])
+def test_emulate_ring_pcie_wires(oracle, nranks, wire):
+    """RingTransmit is instantiated with the 16-byte-message wires (allreduce.cpp:1150-1163)."""
+    for n in (8 * nranks, 8 * nranks * 15, 8 * nranks * 1237):
+        ins = [oracle.generate(n, 51 + r, DIST_NORMAL, 0.0, 1.0) for r in range(nranks)]
+        want = oracle.rotated(ins)
+        for g, w in GEOMS[:5]:
+            rc, io = oracle.emulate_ring(ins, wire, g, w, seq_no=3)
+            assert rc == 0
+            for r in range(nranks):
+                assert (io[r] == want).all(), (n, g, w, r)
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+@pytest.mark.parametrize("wire", [WIRE_RT64_PCIE, WIRE_RT64_128_PCIE])
+def test_emulate_allgather_ring_is_a_copy(oracle, nranks, wire):
+    """runAllgather (sequential_transmit.hpp:474-516): every output ends up as the
+    concatenation of all inputs, also when a rank's input is its own output slot."""
+    for n in (8, 8 * 15, 8 * 1237, 16384):
+        ins = [oracle.generate(n, 61 + r, DIST_UNIFORM, -2.0, 2.0) for r in range(nranks)]
+        want = oracle.allgather(ins)
+        for g, w in GEOMS[:5]:
+            for alias in (False, True):
+                rc, outs = oracle.emulate_allgather_ring(ins, wire, g, w, seq_no=6, alias_own_slot=alias)
+                assert rc == 0
+                for r in range(nranks):
+                    assert (outs[r] == want).all(), (n, g, w, r, alias)
+
+
+def test_emulators_reject_what_the_reference_cannot_run(oracle):
+    ins = [oracle.generate(64, r, DIST_NORMAL, 0.0, 1.0) for r in range(4)]
+    assert oracle.emulate_parallel(ins, WIRE_RT64_PCIE, 1, 4)[0] == -2     # no 256-byte layout restated
+    assert oracle.emulate_sequential(ins, WIRE_RT64_PCIE, 0, 4)[0] == -3   # empty launch
+    assert oracle.emulate_allgather_ring(ins[:3], WIRE_RT64_PCIE, 1, 4)[0] == -2   # 3 ranks: uint32 wrap
 
 
 @pytest.mark.parametrize("nranks", [4, 8, 16])
