@@ -50,6 +50,29 @@ def test_header_compiles_with_plain_gxx(tmp_path):
     assert r.returncode == 0, r.stdout
 
 
+def test_c_abi_header_is_plain_c99_and_links_from_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 and a C program must
+    link against the library and resolve the host-only entry points."""
+    src = tmp_path / "t.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "vrank_allreduce.h"\n'
+        "int main(void) {\n"
+        "  int algo = -1; size_t work = 0; vr_geometry g;\n"
+        '  if (vr_algo_from_string("bisect", &algo) != VR_OK || algo != VR_ALGO_BISECT) return 1;\n'
+        "  const void *bufs[8]; for (int i = 0; i < 8; ++i) bufs[i] = (const void *)0x1000;\n"
+        "  if (vr_check_allreduce(algo, 8, bufs, 16777216, &work) != VR_OK || work != 4194304) return 2;\n"
+        "  if (vr_launch_geometry(algo, 8, 16777216, &g) != VR_OK || g.steps != 69) return 3;  /* allreduce.hpp:237-248: w = NRanks */\n"
+        '  if (strcmp(vr_strerror(VR_ERR_UNEVEN), "We don\'t support non-even divide yet")) return 4;\n'
+        '  puts("c ok"); return 0;\n}\n')
+    exe = tmp_path / "t"
+    lib_dir = os.path.join(ROOT, "gpu_ipc_example_amd")
+    r = run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+             str(src), "-o", str(exe), "-L", lib_dir, "-lvrank_allreduce", "-Wl,-rpath," + lib_dir])
+    assert r.returncode == 0, r.stdout
+    r = run([str(exe)])
+    assert r.returncode == 0 and "c ok" in r.stdout, (r.returncode, r.stdout)
+
+
 @pytest.mark.gpu
 def test_direct_transport_replays_correctly_from_a_hip_graph():
     """A captured small -> copy -> bisect sequence, replayed six times with eager
