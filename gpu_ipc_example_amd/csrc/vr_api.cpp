@@ -865,16 +865,17 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   });
 }
 
-// The probes are pure streaming: nontemporal both ways, large blocks, four
-// 16-byte vectors per lane in flight (what measured best for a plain copy).
-static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, Tuning *t) {
+// The probes are pure streaming: streaming loads, streaming agent-scope stores,
+// four 16-byte vectors per lane in flight.  A 1:1 copy measured best with one
+// 256-lane work-group per CU, the one-way modes with 1024 lanes x 16 waves per CU.
+static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, int mode, Tuning *t) {
   if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
   if (int rc = use_device(ctx)) return rc;
   if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16)
     return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
   Tuning d;
-  d.block = 1024;
-  d.waves_per_cu = 16;
+  d.block = mode == 0 ? 256 : 1024;
+  d.waves_per_cu = mode == 0 ? 4 : 16;
   d.unroll = 4;
   d.nt_load = 1;
   d.nt_store = 2;
@@ -894,7 +895,7 @@ extern "C" int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, c
                                size_t bytes) {
   Tuning t;
   if (mode < 0 || mode > 2) return fail(VR_ERR_INVALID, "bad probe mode");
-  if (int rc = copy_tuning(ctx, dst, src, bytes, &t)) return rc;
+  if (int rc = copy_tuning(ctx, dst, src, bytes, mode, &t)) return rc;
   hipError_t e = launch_copy((hipStream_t)stream, ctx->dev, t, dst, src, bytes, mode);
   return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
 }
@@ -913,7 +914,7 @@ extern "C" int vr_probe_xcc_ids(vr_ctx *ctx, uint32_t blocks, uint32_t *ids_host
 extern "C" int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t bytes,
                             int iters, float *ms_out) {
   Tuning t;
-  if (int rc = copy_tuning(ctx, dst, src, bytes, &t)) return rc;
+  if (int rc = copy_tuning(ctx, dst, src, bytes, 0, &t)) return rc;
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
     hipError_t e = launch_copy(s, ctx->dev, t, dst, src, bytes);
