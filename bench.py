@@ -369,11 +369,11 @@ def main():
         # the same launches on ONE buffer set, with cached instead of streaming loads
         # so that the inputs stay in the memory-side cache
         if not args.tune:
-            ctx.set_tuning(nt_load=0, waves_per_cu=8)
+            ctx.set_tuning(nt_load=0, waves_per_cu=8, f16_wide=0)
         time_kernels(binding, ctx, name, sets[:1], 10)
         wms = time_kernels(binding, ctx, name, sets[:1], 50, group=10)
         if not args.tune:
-            ctx.set_tuning(nt_load=-1, waves_per_cu=-1)
+            ctx.set_tuning(nt_load=-1, waves_per_cu=-1, f16_wide=-1)
         result["same_buffers_cache_warm"] = {
             "GBps": round(B / (float(wms.mean()) * 1e-3) / 1e9, 2),
             "kernel_us_avg": round(float(wms.mean()) * 1e3, 3),

@@ -303,7 +303,10 @@ static hipError_t launch_ar_vec(hipStream_t s, const DeviceInfo &dev, const Tuni
     if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_BF16, h8>(s, dev, t, in, out, bytes);
     return launch_ar_unroll<N, ORDER, DT_BF16, h4>(s, dev, t, in, out, bytes);
   }
-  if (vec_halves == 8) return launch_ar_unroll<N, ORDER, DT_F16, h8>(s, dev, t, in, out, bytes);
+  if (vec_halves == 8) {
+    if (t.f16_wide) return launch_ar_unroll<N, ORDER, DT_F16_WIDE, h8>(s, dev, t, in, out, bytes);
+    return launch_ar_unroll<N, ORDER, DT_F16, h8>(s, dev, t, in, out, bytes);
+  }
   return launch_ar_unroll<N, ORDER, DT_F16, h4>(s, dev, t, in, out, bytes);
 }
 

@@ -174,7 +174,9 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * (persistent grid size = CUs * this / waves per block), "unroll" (16-byte
  * vectors in flight per lane and rank), "nt_load" (0 cached, 1 streaming loads),
  * "nt_store" (0 cached, 1 streaming stores, 2 streaming stores written through
- * at agent scope), "oneshot" (0/1), "segment_kib" (KiB of a chunk one launch
+ * at agent scope), "oneshot" (0/1), "f16_wide" (1 = binary16 adds computed through
+ * binary32 and rounded back after every add: the same bits, a longer ALU section),
+ * "segment_kib" (KiB of a chunk one launch
  * covers; chunks longer than this, at most 1 GiB, take several launches);
  * for the wire transport "wire_fenced" (1 = the Rt64_128 family sends payload
  * lines with a separate flag word ordered by agent-scope release/acquire fences

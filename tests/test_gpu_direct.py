@@ -200,6 +200,42 @@ def test_special_values(ctxs, oracle):
         H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), algo)
 
 
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+def test_adds_through_binary32_give_the_same_bits(ctxs, oracle, nranks):
+    """f16_wide=1 adds binary16 values as binary32 and rounds back after every add:
+    every finite exponent, subnormals, signed zeros, overflow to infinity and
+    inf - inf must come out as from the native binary16 add."""
+    ctx = ctxs[nranks]
+    rng = np.random.default_rng(12 + nranks)
+    n = nranks * 8 * 8192
+    ins = []
+    for r in range(nranks):
+        a = rng.integers(0, 0x10000, n, dtype=np.uint32).astype(np.uint16)
+        a[(a & 0x7C00) == 0x7C00] &= 0x83FF
+        ins.append(a)
+    ins[0][:64] = 0x0001
+    ins[1][:64] = 0x8001
+    ins[0][64:128] = 0x7BFF
+    ins[1][64:128] = 0x7BFF
+    ins[0][128:192] = 0x7C00
+    ins[1][128:192] = 0xFC00
+    ins[0][192:256] = 0x8000                           # -0 + -0 stays -0
+    ins[1][192:256] = 0x8000
+    for r in range(2, nranks):
+        ins[r][:256] = 0x8000
+    small = [oracle.generate(n, 900 + r, DIST_NORMAL, 0.0, 1e-4) for r in range(nranks)]   # sums in the subnormal range
+    ctx.set_tuning(f16_wide=1)
+    try:
+        for data in (ins, small):
+            for algo in ("simple", "bisect") if nranks >= 4 else ("simple",):
+                for unroll in (1, 2):
+                    ctx.set_tuning(unroll=unroll)
+                    got, _ = H.run_allreduce(ctx, algo, data)
+                    H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, data), "%s unroll %d" % (algo, unroll))
+    finally:
+        ctx.set_tuning(f16_wide=-1, unroll=-1)
+
+
 # ---- the five benchmark configurations at full size ------------------------------------------------------
 
 def test_config1_two_ranks_simple(ctxs, oracle):
