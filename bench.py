@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0
 # see profiles/.  Keyed by workload name.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/direct_allreduce_bisect_8x32MiB_hbm_traffic.md
-    "cfg3": 536899583,
+    "cfg3": 536914021,
     # profiles/direct_allgather_4x8MiB_kernel_trace.md
     "cfg4": 167799218,
 }
