@@ -151,6 +151,8 @@ def cpu_leg(name, gpu_results, budget_s):
         host = [o.generate_dt(DTYPE, ne, seed + r, dist, p0, p1) for r in range(n)]
         if algo.startswith("allgather"):
             return host, o.allgather
+        if DTYPE == 0:                      # the oracle's vectorised binary16 loop
+            return host, (o.bisect if algo == "bisect" else o.rotated)
         mode = oracle_lib.ORDER_BISECT if algo == "bisect" else oracle_lib.ORDER_ROTATED
         return host, (lambda ins: o.order_dt(DTYPE, mode, ins))
 
