@@ -548,9 +548,10 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     t.waves_per_cu = 32;
     t.nt_load = 0;
     t.nt_store = 2;
-  } else if (a->latency_tuned) {
-    // "small" family: every lane makes one trip; results stay cacheable for the
-    // kernel that consumes them next.
+  } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) <= kMall) {
+    // "small" family at the sizes it is meant for: every lane makes one trip;
+    // results stay cacheable for the kernel that consumes them next.  (Beyond the
+    // cache it streams like the other protocols.)
     t.waves_per_cu = 8;
     t.oneshot = 1;
     t.nt_load = 0;
