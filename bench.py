@@ -39,6 +39,7 @@ DTYPE_NAMES = {0: "f16", 1: "bf16"}
 
 WORKLOADS = {
     # name: (nranks, algo, nelems per rank, dist, p0, p1, seed)
+    "cfg1": (2, "simple", 16384, 0, -1.0, 1.0, 1000),
     "cfg2": (8, "small", 524288, 1, 0.0, 1.0, 2000),
     "cfg3": (8, "bisect", 16777216, 1, 0.0, 0.02, 3000),
     "cfg4": (4, "allgather_simple", 4194304, 0, -2.0, 2.0, 4000),
