@@ -67,7 +67,10 @@ def lib():
     sig = {
         "vr_ctx_create": (i, [i, i, vpp]),
         "vr_ctx_destroy": (i, [vp]),
+        "vr_ctx_reserve_wire": (i, [vp]),
         "vr_ctx_nranks": (i, [vp]),
+        "vr_allreduce_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
+        "vr_rank_scratch_bytes": (i, [vp, C.POINTER(sz)]),
         "vr_ctx_set_dtype": (i, [vp, i]),
         "vr_ctx_get_dtype": (i, [vp]),
         "vr_fill_pattern_dt": (None, [i, C.POINTER(C.c_uint16), i, sz]),
@@ -242,31 +245,48 @@ class VirtualRanks:
     def set_dtype(self, dtype):
         _check(lib().vr_ctx_set_dtype(self._h, dtype))
 
-    def set_tuning(self, **kw):
-        for k, v in kw.items():
-            _check(lib().vr_ctx_set_tuning(self._h, k.encode(), int(v)))
+    def reserve_wire(self):
+        """Allocate and zero the wire transport's scratch (idempotent)."""
+        _check(lib().vr_ctx_reserve_wire(self._h))
 
-    def get_tuning(self, key):
-        v = C.c_int(0)
-        _check(lib().vr_ctx_get_tuning(self._h, key.encode(), C.byref(v)))
-        return v.value
+    def _reserve_for(self, algo, transport):
+        # The C ABI never allocates inside a collective call; this wrapper reserves
+        # the scratch on the first call that will take the wire transport.
+        if transport == TRANSPORT_WIRE or (transport == TRANSPORT_DEFAULT and algo == "parallel"):
+            self.reserve_wire()
 
-    def set_spin_limit(self, polls):
-        _check(lib().vr_ctx_set_spin_limit(self._h, polls))
+    def rank_scratch_bytes(self):
+        out = C.c_size_t(0)
+        _check(lib().vr_rank_scratch_bytes(self._h, C.byref(out)))
+        return out.value
+
+    def allreduce_rank(self, algo, rank, inp, scatter, gather, peers0, peers1, sink_bytes, nelems,
+                       seq_no, out=None, stream=None):
+        """One rank's wires against caller-owned sinks; returns the advanced sequence number."""
+        seq = C.c_uint32(seq_no)
+        _check(lib().vr_allreduce_rank(self._h, stream, algo_id(algo), rank, C.c_void_p(int(inp)),
+                                       C.c_void_p(int(out)) if out else None,
+                                       C.c_void_p(int(scatter)), C.c_void_p(int(gather)),
+                                       _table(peers0), _table(peers1), sink_bytes, nelems,
+                                       C.byref(seq)))
+        return seq.value
 
     def allreduce(self, algo, bufs, nelems, outs=None, transport=TRANSPORT_DEFAULT, stream=None):
         assert len(bufs) == self.nranks
+        self._reserve_for(algo, transport)
         _check(lib().vr_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
                                   _table(outs) if outs is not None else None, nelems,
                                   C.byref(self.seq_no)))
 
     def allreduce_grid(self, algo, bufs, nelems, groups, subgroups, simd=16, outs=None,
                        transport=TRANSPORT_DEFAULT, stream=None, seq_no=0xE00F100F):
+        self._reserve_for(algo, transport)
         _check(lib().vr_allreduce_grid(self._h, stream, algo_id(algo), transport, _table(bufs),
                                        _table(outs) if outs is not None else None, nelems, seq_no,
                                        groups, subgroups, simd))
 
     def allgather(self, algo, inputs, outputs, nelems, transport=TRANSPORT_DEFAULT, stream=None):
+        self._reserve_for(algo, transport)
         _check(lib().vr_allgather(self._h, stream, algo_id(algo), transport, _table(inputs),
                                   _table(outputs), nelems, C.byref(self.seq_no)))
 
@@ -279,6 +299,7 @@ class VirtualRanks:
     def time_allreduce(self, algo, bufs, nelems, iters, outs=None, transport=TRANSPORT_DEFAULT,
                        stream=None):
         ms = (C.c_float * iters)()
+        self._reserve_for(algo, transport)
         _check(lib().vr_time_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
                                        _table(outs) if outs is not None else None, nelems, iters, ms))
         return np.frombuffer(ms, np.float32).copy()
@@ -286,6 +307,7 @@ class VirtualRanks:
     def time_allgather(self, algo, inputs, outputs, nelems, iters, transport=TRANSPORT_DEFAULT,
                        stream=None):
         ms = (C.c_float * iters)()
+        self._reserve_for(algo, transport)
         _check(lib().vr_time_allgather(self._h, stream, algo_id(algo), transport, _table(inputs),
                                        _table(outputs), nelems, iters, ms))
         return np.frombuffer(ms, np.float32).copy()

@@ -221,23 +221,38 @@ struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
   int segment_kib = -1, f16_wide = -1;
   int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1, wire_ahead = -1, wire_msg16 = -1;
+  int wire_stream_io = -1;
 };
 
-// Scratch of the wire transport: per virtual rank one scatter and one gather
-// sink plus their flag words (the reference's ipcbuf0 / ipcbuf1, main.cpp:241-251),
-// allocated and zeroed on first use.
-struct WireState {
-  bool ready = false;
+// Where the messages of a wire-transport launch go: every rank's scatter and
+// gather sink (the reference's peerBuf0[] / peerBuf1[], main.cpp:260-269) and what
+// they were sized for.
+struct WireSinks {
   void *scatter[VR_MAX_RANKS] = {}, *gather[VR_MAX_RANKS] = {};
-  void *sflag[VR_MAX_RANKS] = {}, *gflag[VR_MAX_RANKS] = {};
-  uint32_t *status = nullptr;
-  size_t sink_bytes = 0, flag_bytes = 0;
-  uint32_t block_threads = 256;   // 4 wires per work-group
-  uint32_t blocks_per_rank_max = 0;
-  bool used = false;              // a launch has written flags since the last clear
-  uint32_t next_min_seq = 0;      // smallest flag value the next launch may start at
+  wl::Layout layout = {};
+  uint32_t wpr_max = 0;        // wires per rank the sinks hold
+  bool simple_ok = false;      // room for SimpleTransmit's sender sections
+};
+
+// What earlier launches left in a set of sinks.
+struct WireHistory {
+  bool used = false;           // a launch has written flags since the last clear
+  uint32_t next_min_seq = 0;   // smallest flag value the next launch may start at
   int last_flow = -1, last_fmt = -1;
 };
+
+// Scratch of the wire transport owned by a context: ONE allocation holding, per
+// virtual rank, a scatter sink followed by a gather sink (the reference's
+// ipcbuf0 | ipcbuf1, main.cpp:241-251), made and zeroed by vr_ctx_reserve_wire.
+struct WireState {
+  bool ready = false;
+  void *base = nullptr;
+  size_t bytes = 0;
+  WireSinks sinks;
+  WireHistory hist;
+};
+
+static const uint32_t kWireBlockThreads = 256;   // 4 wires per work-group
 
 struct vr_ctx {
   int nranks = 0;
@@ -246,6 +261,7 @@ struct vr_ctx {
   uint32_t seq_no = 1;
   uint64_t spin_limit = 0;
   DType dtype = DT_F16;
+  uint32_t *status = nullptr;     // time-out word of this context's wire launches (256 B)
   WireState wire;
 };
 
@@ -255,80 +271,75 @@ static const uint32_t kWireAhead = 4;
 
 static void wire_free(vr_ctx *c) {
   WireState &w = c->wire;
-  for (int r = 0; r < VR_MAX_RANKS; ++r) {
-    if (w.scatter[r]) (void)hipFree(w.scatter[r]);
-    if (w.gather[r]) (void)hipFree(w.gather[r]);
-    if (w.sflag[r]) (void)hipFree(w.sflag[r]);
-    if (w.gflag[r]) (void)hipFree(w.gflag[r]);
-  }
-  if (w.status) (void)hipFree(w.status);
+  if (w.base) (void)hipFree(w.base);
   w = WireState();
 }
 
-static int wire_allocate(vr_ctx *c);
-
-static int wire_prepare(vr_ctx *c) {
-  if (c->wire.ready) return VR_OK;
-  const int rc = wire_allocate(c);
-  if (rc != VR_OK) {          // do not keep a half-built scratch set around
-    const std::string detail = g_detail;
-    wire_free(c);
-    g_detail = detail;
-  }
-  return rc;
+// Wires per rank the context's launches may use: a few 256-lane work-groups per
+// CU (default two; a CU holds eight of them) keep every wire of every rank
+// co-resident.
+static uint32_t wire_wpr_max(const vr_ctx *c) {
+  const int per_cu = c->tune.wire_blocks_per_cu > 0 ? c->tune.wire_blocks_per_cu : kWireBlocksPerCu;
+  uint32_t blocks = (uint32_t)(c->dev.cus * per_cu / c->nranks);
+  if (blocks == 0) blocks = 1;
+  return blocks * (kWireBlockThreads / 64);
 }
 
-static int wire_allocate(vr_ctx *c) {
-  WireState &w = c->wire;
-  HIP_TRY(hipSetDevice(c->dev.device));
-  const int N = c->nranks;
-  // A few 256-lane work-groups per CU (default one; a CU holds eight of them)
-  // keep every wire of every rank co-resident.
-  const int per_cu = c->tune.wire_blocks_per_cu > 0 ? c->tune.wire_blocks_per_cu : kWireBlocksPerCu;
-  w.blocks_per_rank_max = (uint32_t)(c->dev.cus * per_cu / N);
-  if (w.blocks_per_rank_max == 0) w.blocks_per_rank_max = 1;
-  const size_t wpr_max = (size_t)w.blocks_per_rank_max * (w.block_threads / 64);
-  // Slots a sink must hold: ring / sequential / all-gather index [peer][wire] with
-  // 4 slots each; parallel indexes [wire + rank] and bisect [close wires + N/2 |
-  // far wires], both with 8 slots.
-  const size_t slots_ring = 4 * (size_t)N * wpr_max;
-  const size_t slots_flat = (size_t)kWireMaxSlots * (2 * wpr_max + (size_t)N);
-  // SimpleTransmit: one 2 MiB ring section per sender.
-  const size_t slots_simple = (size_t)N * (kSimpleSectionBytes / wire_slot_bytes_max());
-  size_t slots = slots_ring > slots_flat ? slots_ring : slots_flat;
-  if (slots_simple > slots) slots = slots_simple;
-  w.sink_bytes = slots * wire_slot_bytes_max();
-  w.flag_bytes = slots * sizeof(uint32_t);
-  for (int r = 0; r < N; ++r) {
-    HIP_TRY(hipMalloc(&w.scatter[r], w.sink_bytes));
-    HIP_TRY(hipMalloc(&w.gather[r], w.sink_bytes));
-    HIP_TRY(hipMalloc(&w.sflag[r], w.flag_bytes));
-    HIP_TRY(hipMalloc(&w.gflag[r], w.flag_bytes));
-    HIP_TRY(hipMemset(w.scatter[r], 0, w.sink_bytes));      // zeroed once, main.cpp:251
-    HIP_TRY(hipMemset(w.gather[r], 0, w.sink_bytes));
-    HIP_TRY(hipMemset(w.sflag[r], 0, w.flag_bytes));
-    HIP_TRY(hipMemset(w.gflag[r], 0, w.flag_bytes));
+static void sinks_at(WireSinks *k, int nranks, char *base, const wl::Layout &l, uint32_t wpr_max,
+                     bool simple_ok) {
+  *k = WireSinks();
+  for (int r = 0; r < nranks; ++r) {
+    k->scatter[r] = base + (size_t)r * l.rank_bytes;
+    k->gather[r] = base + (size_t)r * l.rank_bytes + l.sink_bytes;
   }
-  HIP_TRY(hipMalloc((void **)&w.status, 256));
-  HIP_TRY(hipMemset(w.status, 0, 256));
-  HIP_TRY(hipDeviceSynchronize());
+  k->layout = l;
+  k->wpr_max = wpr_max;
+  k->simple_ok = simple_ok;
+}
+
+extern "C" int vr_ctx_reserve_wire(vr_ctx *c) {
+  if (!c) return fail(VR_ERR_INVALID, "null ctx");
+  WireState &w = c->wire;
+  if (w.ready) return VR_OK;
+  HIP_TRY(hipSetDevice(c->dev.device));
+  const uint32_t wpr_max = wire_wpr_max(c);
+  const wl::Layout l = wl::layout_for(c->nranks, wpr_max, true);
+  w.bytes = (size_t)c->nranks * l.rank_bytes;
+  hipError_t e = hipMalloc(&w.base, w.bytes);
+  if (e == hipSuccess) e = hipMemset(w.base, 0, w.bytes);      // zeroed once, main.cpp:251
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e != hipSuccess) {
+    wire_free(c);
+    return fail_hip(e, "reserving the wire-transport scratch");
+  }
+  sinks_at(&w.sinks, c->nranks, static_cast<char *>(w.base), l, wpr_max, true);
   w.ready = true;
   return VR_OK;
 }
 
-// Forget every flag ever written (asynchronous, ordered on `s`).
-static int wire_clear(vr_ctx *c, hipStream_t s) {
-  WireState &w = c->wire;
-  for (int r = 0; r < c->nranks; ++r) {
-    hipError_t e = launch_wire_clear(s, w.scatter[r], w.sink_bytes);
-    if (e == hipSuccess) e = launch_wire_clear(s, w.gather[r], w.sink_bytes);
-    if (e == hipSuccess) e = launch_wire_clear(s, w.sflag[r], w.flag_bytes);
-    if (e == hipSuccess) e = launch_wire_clear(s, w.gflag[r], w.flag_bytes);
-    if (e != hipSuccess) return fail_hip(e, "launch_wire_clear");
-  }
-  w.used = false;
+extern "C" int vr_rank_scratch_bytes(const vr_ctx *c, size_t *sink_bytes) {
+  if (!c || !sink_bytes) return fail(VR_ERR_INVALID, "null argument");
+  *sink_bytes = wl::layout_for(c->nranks, wire_wpr_max(c), true).sink_bytes;
   return VR_OK;
 }
+
+// Forget every flag ever written (asynchronous, ordered on `s`).
+static int wire_clear(const WireSinks &k, int nranks, hipStream_t s) {
+  for (int r = 0; r < nranks; ++r) {
+    hipError_t e = launch_wire_clear(s, k.scatter[r], k.layout.sink_bytes);
+    if (e == hipSuccess) e = launch_wire_clear(s, k.gather[r], k.layout.sink_bytes);
+    if (e != hipSuccess) return fail_hip(e, "launch_wire_clear");
+  }
+  return VR_OK;
+}
+
+struct WireLaunch {
+  const WireSinks *sinks;
+  WireHistory *hist;      // null: the caller owns the sinks and the sequence numbers (one-rank launches)
+  uint32_t *status;
+  int solo_rank;          // >= 0: launch this rank's wires only
+  bool always_clear;      // clear the sinks before every launch (fixed scratch shared by contexts)
+};
 
 // Launches one wire-transport collective.  `user_wires` (0 = automatic) is the
 // number of sub-groups per rank a caller asked for with -g/-w.  *seq_io is the
@@ -337,46 +348,74 @@ static int wire_clear(vr_ctx *c, hipStream_t s) {
 // through *flags_used how many consecutive flag values the launch consumes.
 static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
                        const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t *seq_io,
-                       uint32_t user_wires, uint32_t *flags_used) {
+                       uint32_t user_wires, uint32_t *flags_used, const WireLaunch &wlch) {
   uint32_t seq = *seq_io;
   if (seq == 0)
     return fail(VR_ERR_INVALID, "sequence number 0 cannot be told from freshly zeroed scratch");
-  if (int rc = wire_prepare(c)) return rc;
-  WireState &w = c->wire;
+  const WireSinks &k = *wlch.sinks;
   const int N = c->nranks;
   const WireFlow flow = a->wire_flow();
   WireFormat fmt = a->wire_format();
   if (fmt == WIRE_FMT_LL64 && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
   if (fmt == WIRE_FMT_LL16 && c->tune.wire_msg16 == 0) fmt = WIRE_FMT_LL;
+  if (flow == WIRE_SIMPLE && !k.simple_ok)
+    return fail(VR_ERR_INVALID, "these sinks have no room for SimpleTransmit's 2 MiB sender sections");
+  // The flag values of a launch are kernel arguments, and whether the sinks must
+  // be cleared first is decided here on the host: a captured launch would replay
+  // with stale flags.  (With always_clear every replay starts from clean sinks.)
+  if (!wlch.always_clear) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(VR_ERR_INVALID, "the wire transport cannot be captured into a graph: its flag values "
+                                  "are per-launch kernel arguments (capture the direct transport)");
+    (void)hipGetLastError();
+  }
   const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
-  const uint32_t waves_per_block = w.block_threads / 64;
-  const uint32_t wpr_limit = w.blocks_per_rank_max * waves_per_block / psg * psg;
-  if (wpr_limit < psg) return fail(VR_ERR_INVALID, "device too small for this rank count");
+  const uint32_t waves_per_block = kWireBlockThreads / 64;
+  const uint32_t wpr_limit = k.wpr_max / psg * psg;
+  if (wpr_limit < psg) return fail(VR_ERR_INVALID, "sinks too small for this rank count");
   const uint32_t wire_bytes = wire_bytes_per_step(fmt, vec_halves);
   const size_t wires_per_chunk = div_up(chunk_bytes, wire_bytes);
   if (wires_per_chunk == 0) { *flags_used = 0; return VR_OK; }
   size_t want = user_wires ? (size_t)user_wires / psg * psg : wires_per_chunk * psg;
   if (want < psg) want = psg;
   if (want > wpr_limit) want = wpr_limit;
-  // SimpleTransmit's ring sections hold 2 MiB of messages per sender; a sender
-  // runs at most one step ahead of its receivers, so two steps must fit.
-  const size_t per_section = kSimpleSectionBytes / wire_slot_bytes_max();
-  if (flow == WIRE_SIMPLE && want > per_section / 2) want = per_section / 2;
+  if (flow == WIRE_SIMPLE) {
+    // A sender runs at most one step ahead of its receivers, so two steps must fit
+    // a section; and only a power of two divides the section, which keeps every
+    // ring position with the wave that used it before.
+    if (want > wl::kSimplePerSection / 2) want = wl::kSimplePerSection / 2;
+    size_t pow2 = 1;
+    while (pow2 * 2 <= want) pow2 *= 2;
+    want = pow2;
+  }
   const uint32_t wpr = (uint32_t)want;
+  if (wl::slots_needed((int)flow, N, wpr) > k.layout.slots)
+    return fail(VR_ERR_INVALID, "internal: sink smaller than the flow's slot range");
   const uint32_t blocks_per_rank = (uint32_t)div_up(wpr, waves_per_block);
   const size_t steps = div_up(wires_per_chunk, wpr / psg);
   const uint32_t nslot_min = 4;
-  *flags_used = flow == WIRE_SIMPLE ? (uint32_t)(steps * wpr / per_section + 1)
+  *flags_used = flow == WIRE_SIMPLE ? (uint32_t)(steps * wpr / wl::kSimplePerSection + 1)
                                     : (uint32_t)((steps - 1) / nslot_min + 1);
 
   // Flags must strictly increase on every slot and never be 0 (the value of
   // cleared scratch); a different flow or format re-interprets the sinks.  In all
   // those cases start from a clean slate.
   const bool wraps = (uint32_t)(seq + *flags_used) < seq;
+  if (wraps && !wlch.hist && !wlch.always_clear)
+    return fail(VR_ERR_INVALID, "the sequence number would wrap through 0: zero every rank's scratch "
+                                "and restart from 1");
   if (wraps) seq = 1;
-  const bool moved_back = w.used && (int32_t)(seq - w.next_min_seq) < 0;
-  if (wraps || moved_back || (w.used && (w.last_flow != (int)flow || w.last_fmt != (int)fmt)))
-    if (int rc = wire_clear(c, s)) return rc;
+  if (wlch.always_clear) {
+    if (int rc = wire_clear(k, N, s)) return rc;
+  } else if (wlch.hist) {
+    WireHistory &h = *wlch.hist;
+    const bool moved_back = h.used && (int32_t)(seq - h.next_min_seq) < 0;
+    if (wraps || moved_back || (h.used && (h.last_flow != (int)flow || h.last_fmt != (int)fmt))) {
+      if (int rc = wire_clear(k, N, s)) return rc;
+      h.used = false;
+    }
+  }
   *seq_io = seq;
 
   WireArgs args;
@@ -384,27 +423,47 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   args.in = in;
   args.out = out;
   for (int r = 0; r < N; ++r) {
-    args.scatter.p[r] = w.scatter[r];
-    args.gather.p[r] = w.gather[r];
-    args.sflag.p[r] = w.sflag[r];
-    args.gflag.p[r] = w.gflag[r];
+    args.scatter.p[r] = k.scatter[r];
+    args.gather.p[r] = k.gather[r];
   }
+  args.flag_off = k.layout.flag_off;
   args.chunk_bytes = chunk_bytes;
   args.waves_per_rank = wpr;
   args.seq = seq;
   const uint64_t limit = c->spin_limit ? c->spin_limit : kDefaultSpinLimit;
   args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
-  args.status = w.status;
+  args.status = wlch.status;
   args.ahead = c->tune.wire_ahead > 0 ? (uint32_t)c->tune.wire_ahead : kWireAhead;
-  const bool cooperative = c->tune.wire_cooperative != 0;
-  hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks_per_rank, w.block_threads, args,
-                             cooperative, c->dtype);
-  if (e != hipSuccess) return fail_hip(e, cooperative ? "launch_wire (cooperative)" : "launch_wire");
-  w.used = true;
-  w.next_min_seq = seq + *flags_used;
-  w.last_flow = (int)flow;
-  w.last_fmt = (int)fmt;
+  args.solo_rank = wlch.solo_rank;
+  // Cached accesses measured faster than streaming ones for the wires' narrow
+  // per-lane inputs and outputs (a write-through store of part of a line costs a
+  // read-modify-write at the memory side); streaming stays selectable.
+  args.stream_io = c->tune.wire_stream_io > 0 ? 1u : 0u;
+  const bool solo = wlch.solo_rank >= 0;
+  // One rank's launch cannot vouch for the other ranks' work-groups: plain launch.
+  const int cooperative = solo ? 0 : c->tune.wire_cooperative;
+  const uint32_t blocks = solo ? blocks_per_rank : blocks_per_rank * (uint32_t)N;
+  hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks, kWireBlockThreads, args,
+                             cooperative, c->dev.cus, c->dtype);
+  if (e != hipSuccess) return fail_hip(e, "launch_wire");
+  if (wlch.hist) {
+    wlch.hist->used = true;
+    wlch.hist->next_min_seq = seq + *flags_used;
+    wlch.hist->last_flow = (int)flow;
+    wlch.hist->last_fmt = (int)fmt;
+  }
   return VR_OK;
+}
+
+// Launch on the context's own scratch.
+static int wire_launch_ctx(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
+                           const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t *seq_io,
+                           uint32_t user_wires, uint32_t *flags_used) {
+  if (!c->wire.ready)
+    return fail(VR_ERR_INVALID, "the wire transport's scratch is not reserved: call "
+                                "vr_ctx_reserve_wire(ctx) once before the first wire-transport launch");
+  const WireLaunch wlch = {&c->wire.sinks, &c->wire.hist, c->status, -1, false};
+  return wire_launch(c, s, a, in, out, chunk_bytes, vec_halves, seq_io, user_wires, flags_used, wlch);
 }
 
 
@@ -424,11 +483,20 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(VR_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", kernels are built for gfx950");
   HIP_TRY(hipSetDevice(device));
+  // Set-up work that must not happen in a hot call: the context's time-out word.
+  uint32_t *status = nullptr;
+  HIP_TRY(hipMalloc((void **)&status, 256));
+  hipError_t e = hipMemset(status, 0, 256);
+  if (e != hipSuccess) {
+    (void)hipFree(status);
+    return fail_hip(e, "vr_ctx_create set-up");
+  }
   vr_ctx *c = new vr_ctx;
   c->nranks = nranks;
   c->dev.device = device;
   c->dev.cus = prop.multiProcessorCount;
   snprintf(c->dev.arch, sizeof c->dev.arch, "%s", prop.gcnArchName);
+  c->status = status;
   *out = c;
   return VR_OK;
 }
@@ -436,6 +504,7 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
 extern "C" int vr_ctx_destroy(vr_ctx *ctx) {
   if (!ctx) return VR_OK;
   wire_free(ctx);
+  if (ctx->status) (void)hipFree(ctx->status);
   delete ctx;
   return VR_OK;
 }
@@ -472,6 +541,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
   if (!strcmp(key, "wire_ahead")) return &ctx->tune.wire_ahead;
   if (!strcmp(key, "wire_msg16")) return &ctx->tune.wire_msg16;
+  if (!strcmp(key, "wire_stream_io")) return &ctx->tune.wire_stream_io;
   return nullptr;
 }
 
@@ -485,7 +555,7 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
     if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
       return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
-    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") || !strcmp(key, "wire_msg16") || !strcmp(key, "f16_wide") ||
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") || !strcmp(key, "wire_msg16") || !strcmp(key, "f16_wide") || !strcmp(key, "wire_stream_io") ||
          !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
@@ -497,7 +567,7 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "wire_ahead must be in [1,6]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
       if (value < 1 || value > 4) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be in [1,4]");
-      if (ctx->wire.ready) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be set before the first wire-transport launch");
+      if (ctx->wire.ready) return fail(VR_ERR_INVALID, "wire_blocks_per_cu must be set before vr_ctx_reserve_wire");
     }
   }
   *f = value;
@@ -650,10 +720,11 @@ static int run_allreduce(vr_ctx *ctx, hipStream_t s, const Prepared &p, int tran
                          const Tuning &t, uint32_t seq_no, uint32_t user_wires, uint32_t *next_seq) {
   uint32_t advance = p.geom.steps;  // getLaunchParam: updateSeqNo += nSteps
   *next_seq = seq_no + advance;
+  if (*next_seq == 0) *next_seq = 1;   // 0 is the value of cleared scratch: never hand it out
   if (transport == VR_TRANSPORT_WIRE) {
     uint32_t used = 0;
-    if (int rc = wire_launch(ctx, s, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, &seq_no,
-                             user_wires, &used))
+    if (int rc = wire_launch_ctx(ctx, s, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, &seq_no,
+                                 user_wires, &used))
       return rc;
     if (used > advance) advance = used;
     *next_seq = seq_no + advance;
@@ -712,6 +783,68 @@ extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transp
                        wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &next);
 }
 
+// One rank of an all-reduce, the form the reference constructs per process
+// (allreduce.hpp:18-28, parallel_transmit.hpp:36-60, bisect_transmit.hpp:427-482).
+extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
+                                 void *output, void *scatter_buf, void *gather_buf,
+                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
+                                 size_t nelems, uint32_t *seq_no) {
+  if (int rc = use_device(ctx)) return rc;
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
+  const int N = ctx->nranks;
+  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!seq_no) return fail(VR_ERR_INVALID, "a one-rank launch needs the caller's sequence number");
+  if (!scatter_buf || !gather_buf || !peer_buf0 || !peer_buf1)
+    return fail(VR_ERR_INVALID, "null scratch pointer");
+  if (!output) output = input;
+  // calcWorkSize sees this rank's pointers only (allreduce.hpp:108-122).
+  const void *table[VR_MAX_RANKS];
+  for (int r = 0; r < N; ++r) table[r] = input;
+  size_t work = 0;
+  if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
+  for (int r = 0; r < N; ++r) table[r] = output;
+  if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
+  if (ranges_partially_overlap(output, input, nelems * 2))
+    return fail(VR_ERR_OVERLAP, "output partially overlaps input");
+  const uint32_t wpr_max = wire_wpr_max(ctx);
+  const wl::Layout l = wl::layout_for(N, wpr_max, true);
+  if (sink_bytes < l.sink_bytes)
+    return fail(VR_ERR_INVALID, "sinks hold " + std::to_string(sink_bytes) + " bytes, this context needs " +
+                                    std::to_string(l.sink_bytes) + " (vr_rank_scratch_bytes)");
+  WireSinks k;
+  k.layout = l;
+  k.wpr_max = wpr_max;
+  k.simple_ok = true;
+  for (int r = 0; r < N; ++r) {
+    k.scatter[r] = r == rank ? scatter_buf : peer_buf0[r];
+    k.gather[r] = r == rank ? gather_buf : peer_buf1[r];
+    if (!k.scatter[r] || !k.gather[r]) return fail(VR_ERR_INVALID, "null peer sink for rank " + std::to_string(r));
+    if ((uintptr_t)k.scatter[r] % 16 || (uintptr_t)k.gather[r] % 16)
+      return fail(VR_ERR_UNALIGNED, "sinks must be 16-byte aligned");
+  }
+  PtrTable in, out;
+  memset(&in, 0, sizeof in);
+  memset(&out, 0, sizeof out);
+  in.p[rank] = input;
+  out.p[rank] = output;
+  const size_t chunk_elems = work / 2;
+  const bool align16 = (uintptr_t)input % 16 == 0 && (uintptr_t)output % 16 == 0;
+  // Every rank must pick the same message shape; only the fenced format depends on
+  // the access width, and there the caller's buffers decide it for all ranks.
+  const int vec_halves = (align16 && chunk_elems % 8 == 0) ? 8 : 4;
+  vr_geometry geom;
+  if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
+  const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};
+  uint32_t seq = *seq_no, used = 0;
+  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, chunk_elems * 2, vec_halves, &seq, 0,
+                           &used, wlch))
+    return rc;
+  *seq_no = seq + (used > geom.steps ? used : geom.steps);
+  if (*seq_no == 0) *seq_no = 1;
+  return VR_OK;
+}
+
 struct PreparedGather {
   const AlgoInfo *a;
   PtrTable in, out;
@@ -762,8 +895,8 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
   if (transport == VR_TRANSPORT_WIRE) {
     uint32_t used = 0, start = *seq;
-    if (int rc = wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start,
-                             0, &used))
+    if (int rc = wire_launch_ctx(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves,
+                                 &start, 0, &used))
       return rc;
     *seq = start + (used > p.geom.steps ? used : p.geom.steps);
     if (*seq == 0) *seq = 1;
@@ -776,23 +909,36 @@ extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
                                          ctx->nranks, p.in, p.out, nelems, p.vec_halves);
   if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
   *seq += p.geom.steps;
+  if (*seq == 0) *seq = 1;
+  return VR_OK;
+}
+
+// Reads one time-out word; if set, resets it and reports the time-out.
+static int check_status_word(uint32_t *word, bool *timed_out) {
+  uint32_t status = 0;
+  HIP_TRY(hipMemcpy(&status, word, sizeof status, hipMemcpyDeviceToHost));
+  if (status != 0) {
+    HIP_TRY(hipMemset(word, 0, sizeof status));
+    *timed_out = true;
+  }
   return VR_OK;
 }
 
 extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
   if (int rc = use_device(ctx)) return rc;
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  WireState &w = ctx->wire;
-  if (!w.ready) return VR_OK;
-  uint32_t status = 0;
-  HIP_TRY(hipMemcpy(&status, w.status, sizeof status, hipMemcpyDeviceToHost));
-  if (status == 0) return VR_OK;
-  // A poll gave up: results of that launch are undefined and half-delivered
-  // messages may still sit in the sinks.  Start over from clean scratch.
-  HIP_TRY(hipMemset(w.status, 0, 256));
-  if (int rc = wire_clear(ctx, (hipStream_t)stream)) return rc;
-  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  return fail(VR_ERR_TIMEOUT, "a wire-transport poll exceeded the spin limit; scratch was reset");
+  bool timed_out = false;
+  if (int rc = check_status_word(ctx->status, &timed_out)) return rc;
+  if (timed_out && ctx->wire.ready) {
+    // A poll gave up: results of that launch are undefined and half-delivered
+    // messages may still sit in the sinks.  Start over from clean scratch.
+    if (int rc = wire_clear(ctx->wire.sinks, ctx->nranks, (hipStream_t)stream)) return rc;
+    ctx->wire.hist.used = false;
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  }
+  if (timed_out)
+    return fail(VR_ERR_TIMEOUT, "a wire-transport poll exceeded the spin limit; scratch was reset");
+  return VR_OK;
 }
 
 // ---------------------------------------------------------------------------------
@@ -862,7 +1008,7 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   return time_launches(s, iters, ms_out, [&]() -> int {
     if (transport == VR_TRANSPORT_WIRE) {
       uint32_t used = 0, start = ctx->seq_no;
-      int rc = wire_launch(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start, 0, &used);
+      int rc = wire_launch_ctx(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start, 0, &used);
       ctx->seq_no = start + (used > p.geom.steps ? used : p.geom.steps);
       if (ctx->seq_no == 0) ctx->seq_no = 1;
       return rc;

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "vrank_allreduce.h"
+#include "vr_wire_layout.h"
 
 namespace vr {
 
@@ -67,7 +68,6 @@ hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device
 
 // Wire transport ------------------------------------------------------------------
 enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER, WIRE_SIMPLE };
-constexpr uint32_t kSimpleSectionBytes = 0x200000;   // simple_transmit.hpp:11
 enum WireFormat : int {
   WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
   WIRE_FMT_LL64 = 1,  // 60 B payload + 4 B flag per 64-byte segment (Rt64_128 family)
@@ -77,23 +77,26 @@ enum WireFormat : int {
 constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
 
 struct WireArgs {
-  PtrTable in, out;          // per-rank input / output
-  PtrTable scatter, gather;  // per-rank sinks
-  PtrTable sflag, gflag;     // per-rank flag words (WIRE_FMT_FLAG)
+  PtrTable in, out;          // per-rank input / output (a one-rank launch fills only its own entry)
+  PtrTable scatter, gather;  // per-rank sinks (the reference's peerBuf0[] / peerBuf1[])
+  size_t flag_off;           // byte offset of the flag words inside a sink (WIRE_FMT_FLAG)
   size_t chunk_bytes;        // bytes per rank-chunk (all-gather: bytes of one slice)
   uint32_t waves_per_rank;   // wires each virtual rank runs (multiple of the flow's waves per column)
   uint32_t seq;              // first flag value of this launch
   uint32_t spin_limit;
   uint32_t ahead;            // steps the scatters of the parallel flow run ahead of its gathers
+  int solo_rank;             // >= 0: the grid holds this one rank's wires only; -1: block b is rank b % N
+  uint32_t stream_io;        // 1: inputs are loaded and outputs stored with streaming cache policies
   uint32_t *status;          // non-zero once any poll gave up
 };
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves);
-uint32_t wire_slot_bytes_max();
-// cooperative: hipLaunchCooperativeKernel instead of a plain launch.
+// Chooses a plain launch when the occupancy query proves that `blocks` work-groups
+// of the flow's kernel are co-resident on `cus` compute units, a cooperative
+// launch otherwise.  cooperative: -1 automatic, 0 plain, 1 cooperative.
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
-                       bool cooperative, DType dtype);
+                       uint32_t blocks, uint32_t block_threads, WireArgs &args,
+                       int cooperative, int cus, DType dtype);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
 
 

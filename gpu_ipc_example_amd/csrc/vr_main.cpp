@@ -176,14 +176,14 @@ int main(int argc, char **argv) try {
   auto run = [&](uint32_t flag) {
     uint32_t step = flag;
     if (gather) {
-      vrank::check(vr_allgather(ranks.get(), stream, algo, ranks.transport(),
+      vrank::check(vr_allgather(ranks.get(), stream, algo, ranks.transportFor(algo),
                                 (const void *const *)input.data(), output.data(), nelems, &step));
     } else if (o.grid_given) {
-      vrank::check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transport(), input.data(),
+      vrank::check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transportFor(algo), input.data(),
                                      nullptr, nelems, flag, (uint32_t)o.groups,
                                      (uint32_t)o.subgroups, o.simd));
     } else {
-      vrank::check(vr_allreduce(ranks.get(), stream, algo, ranks.transport(), input.data(), nullptr,
+      vrank::check(vr_allreduce(ranks.get(), stream, algo, ranks.transportFor(algo), input.data(), nullptr,
                                 nelems, &step));
     }
   };

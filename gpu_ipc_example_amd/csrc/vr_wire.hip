@@ -1,7 +1,9 @@
 // Wire transport: the reference's message-passing stage structure on one GPU.
 //
-// One persistent, cooperatively launched kernel holds the work-groups of ALL
-// virtual ranks (block b belongs to rank b % N).  A wavefront plays the part of
+// One persistent kernel holds the work-groups of ALL virtual ranks (block b
+// belongs to rank b % N), or, launched once per rank (WireArgs::solo_rank), the
+// work-groups of one rank only, as one process per GPU would run it.  A
+// wavefront plays the part of
 // a reference sub-group ("wire"): it loads its rank's input, pushes messages
 // into peers' scatter/gather sinks in device scratch, polls its own sinks, adds
 // in the reference's order and stores.  Sink indexing, slot rotation and flag
@@ -36,6 +38,55 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 
 #define VR_AGENT __HIP_MEMORY_SCOPE_AGENT
 
+// Cache-policy operand of the buffer instructions: bit 1 = nt, bit 4 = sc1.
+constexpr int kIoCached = 0;
+constexpr int kIoStreamLoad = 2;        // nt
+constexpr int kIoStreamStore = 2 | 16;  // nt sc1: streaming, written through at agent scope
+
+// Inputs and outputs are addressed through a buffer resource over the bytes that
+// remain of the chunk at the wire's offset: the hardware returns zero for loads
+// and drops stores at or beyond that length, which is the per-lane predicate of
+// the reference's tail wire (rt64_128.hpp:570-582).  The wire's address and
+// length depend on the wave's index only; saying so keeps the resource in scalar
+// registers.
+static __device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_rsrc(const void *p, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  // (the builtin returns int: go through uint32_t, or a low half with bit 31 set
+  // would sign-extend into the high half)
+  const uint64_t u = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                     ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+  const int n = __builtin_amdgcn_readfirstlane((int)bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char *>(u), 0, n, 0x00020000);
+}
+
+typedef unsigned int io_u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int io_u32x4 __attribute__((ext_vector_type(4)));
+
+static __device__ __forceinline__ uint32_t io_ld32(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
+  return nt ? __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoStreamLoad)
+            : __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoCached);
+}
+static __device__ __forceinline__ io_u32x2 io_ld64(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
+  return nt ? __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoStreamLoad)
+            : __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoCached);
+}
+static __device__ __forceinline__ io_u32x4 io_ld128(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
+  return nt ? __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoStreamLoad)
+            : __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoCached);
+}
+static __device__ __forceinline__ void io_st32(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t v, bool nt) {
+  if (nt) __builtin_amdgcn_raw_buffer_store_b32(v, rs, off, 0, kIoStreamStore);
+  else __builtin_amdgcn_raw_buffer_store_b32(v, rs, off, 0, kIoCached);
+}
+static __device__ __forceinline__ void io_st64(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x2 v, bool nt) {
+  if (nt) __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kIoStreamStore);
+  else __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kIoCached);
+}
+static __device__ __forceinline__ void io_st128(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x4 v, bool nt) {
+  if (nt) __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kIoStreamStore);
+  else __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kIoCached);
+}
+
 struct Spin {
   uint32_t limit;
   uint32_t *status;
@@ -65,21 +116,18 @@ struct WireLL {
     uint32_t d[U];
   };
 
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
     Reg r;
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t off = (u * 64u + lane) * 4u;
-      r.d[u] = off < left ? *reinterpret_cast<const uint32_t *>(p + off) : 0u;
-    }
+    for (int u = 0; u < U; ++u) r.d[u] = io_ld32(rs, (u * 64u + lane) * 4u, nt);
     return r;
   }
-  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
+                                               bool nt) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint32_t off = (u * 64u + lane) * 4u;
-      if (off < left) *reinterpret_cast<uint32_t *>(p + off) = r.d[u];
-    }
+    for (int u = 0; u < U; ++u) io_st32(rs, (u * 64u + lane) * 4u, r.d[u], nt);
   }
   // v = m + v, element-wise binary16, message on the left (rt64.hpp:452-463).
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
@@ -158,32 +206,28 @@ struct WireLL16 {
   struct Reg {
     uint32_t d[U][2];
   };
-  // A slot address is the same in every lane of a wave (it depends on the wave's
-  // index only); saying so keeps the resource in scalar registers.
+  // A slot address is the same in every lane of a wave.
   static __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const char *slot) {
-    const uint64_t a = reinterpret_cast<uint64_t>(slot);
-    // (the builtin returns int: go through uint32_t, or a low half with bit 31 set
-    // would sign-extend into the high half)
-    const uint64_t u = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
-                       ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
-    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char *>(u), 0, (int)kSlotBytes, 0x00020000);
+    return wave_rsrc(slot, kSlotBytes);
   }
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
     Reg r;
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t off = (u * 64u + lane) * 8u;
-      const uint2 z = off < left ? *reinterpret_cast<const uint2 *>(p + off) : make_uint2(0u, 0u);
+      const io_u32x2 z = io_ld64(rs, (u * 64u + lane) * 8u, nt);
       r.d[u][0] = z.x;
       r.d[u][1] = z.y;
     }
     return r;
   }
-  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
+                                               bool nt) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t off = (u * 64u + lane) * 8u;
-      if (off < left) *reinterpret_cast<uint2 *>(p + off) = make_uint2(r.d[u][0], r.d[u][1]);
+      const io_u32x2 z = {r.d[u][0], r.d[u][1]};
+      io_st64(rs, (u * 64u + lane) * 8u, z, nt);
     }
   }
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64.hpp:126-134
@@ -268,26 +312,27 @@ struct WireLL64 {
   static __device__ __forceinline__ uint32_t dword0(int u, uint32_t lane) {
     return (uint32_t)u * 120u + (lane >> 3) * 15u + (lane & 7u) * 2u;
   }
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
     Reg r;
-    const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
     const bool two = (lane & 7u) != 7u;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = dword0(u, lane);
-      r.d[u][0] = 4u * i < left ? q[i] : 0u;
-      r.d[u][1] = (two && 4u * (i + 1) < left) ? q[i + 1] : 0u;
+      r.d[u][0] = io_ld32(rs, 4u * i, nt);
+      r.d[u][1] = two ? io_ld32(rs, 4u * (i + 1), nt) : 0u;
     }
     return r;
   }
-  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
-    uint32_t *q = reinterpret_cast<uint32_t *>(p);
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
+                                               bool nt) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
     const bool two = (lane & 7u) != 7u;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = dword0(u, lane);
-      if (4u * i < left) q[i] = r.d[u][0];
-      if (two && 4u * (i + 1) < left) q[i + 1] = r.d[u][1];
+      io_st32(rs, 4u * i, r.d[u][0], nt);
+      if (two) io_st32(rs, 4u * (i + 1), r.d[u][1], nt);
     }
   }
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:947-957
@@ -367,21 +412,25 @@ struct WireFlag {
     V d[U];
   };
 
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
     Reg r;
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
-      V z = {};
-      r.d[u] = off < left ? *reinterpret_cast<const V *>(p + off) : z;
+      if constexpr (sizeof(V) == 16) r.d[u] = __builtin_bit_cast(V, io_ld128(rs, off, nt));
+      else r.d[u] = __builtin_bit_cast(V, io_ld64(rs, off, nt));
     }
     return r;
   }
-  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r) {
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
+                                               bool nt) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
-      if (off < left) *reinterpret_cast<V *>(p + off) = r.d[u];
+      if constexpr (sizeof(V) == 16) io_st128(rs, off, __builtin_bit_cast(io_u32x4, r.d[u]), nt);
+      else io_st64(rs, off, __builtin_bit_cast(io_u32x2, r.d[u]), nt);
     }
   }
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {
@@ -433,30 +482,35 @@ struct WireFlag {
 };
 
 // ---- sinks --------------------------------------------------------------------------
-
-template <typename W, int NSLOT>
+// A rank's scatter / gather sink: message slots of W::kSlotBytes, then (at
+// flag_off) one flag word per slot.  Slot indices come from vr_wire_layout.h.
+template <typename W>
 struct Sinks {
   const WireArgs &a;
-  __device__ __forceinline__ char *scat(int rank, uint32_t entry, uint32_t s) const {
-    return static_cast<char *>(a.scatter.p[rank]) + ((size_t)entry * NSLOT + s) * W::kSlotBytes;
+  __device__ __forceinline__ char *scat(int rank, uint32_t slot) const {
+    return static_cast<char *>(a.scatter.p[rank]) + (size_t)slot * W::kSlotBytes;
   }
-  __device__ __forceinline__ char *gath(int rank, uint32_t entry, uint32_t s) const {
-    return static_cast<char *>(a.gather.p[rank]) + ((size_t)entry * NSLOT + s) * W::kSlotBytes;
+  __device__ __forceinline__ char *gath(int rank, uint32_t slot) const {
+    return static_cast<char *>(a.gather.p[rank]) + (size_t)slot * W::kSlotBytes;
   }
-  __device__ __forceinline__ uint32_t *sflag(int rank, uint32_t entry, uint32_t s) const {
-    return static_cast<uint32_t *>(a.sflag.p[rank]) + (size_t)entry * NSLOT + s;
+  __device__ __forceinline__ uint32_t *sflag(int rank, uint32_t slot) const {
+    return reinterpret_cast<uint32_t *>(static_cast<char *>(a.scatter.p[rank]) + a.flag_off) + slot;
   }
-  __device__ __forceinline__ uint32_t *gflag(int rank, uint32_t entry, uint32_t s) const {
-    return static_cast<uint32_t *>(a.gflag.p[rank]) + (size_t)entry * NSLOT + s;
+  __device__ __forceinline__ uint32_t *gflag(int rank, uint32_t slot) const {
+    return reinterpret_cast<uint32_t *>(static_cast<char *>(a.gather.p[rank]) + a.flag_off) + slot;
   }
 };
 
+// Rank and wire of this wave.  A launch either holds every rank's work-groups
+// (block b belongs to rank b % N) or one rank's only (solo_rank).
 #define VR_WAVE_PROLOGUE                                                             \
-  const int r = blockIdx.x % N;                                                      \
+  const bool solo = a.solo_rank >= 0;                                                \
+  const int r = solo ? a.solo_rank : (int)(blockIdx.x % N);                          \
   const uint32_t lane = threadIdx.x & 63u;                                           \
-  const uint32_t wid = (blockIdx.x / N) * (blockDim.x >> 6) + (threadIdx.x >> 6);    \
+  const uint32_t wid = (solo ? blockIdx.x : blockIdx.x / N) * (blockDim.x >> 6) + (threadIdx.x >> 6); \
   if (wid >= a.waves_per_rank) return;                                               \
   Spin spin{a.spin_limit, a.status, lane, false};                                    \
+  const bool nt = a.stream_io != 0;                                                  \
   const size_t chunk = a.chunk_bytes
 
 static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, uint32_t wire) {
@@ -469,10 +523,10 @@ static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, 
 // the column's reduction for its rank's chunk.
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
-  constexpr int NSLOT = 8;
+  constexpr uint32_t NSLOT = wl::kSlotsFlat;
   const uint32_t kAhead = a.ahead;   // 1 ... NSLOT - 2, checked by the host
   VR_WAVE_PROLOGUE;
-  const Sinks<W, NSLOT> sk{a};
+  const Sinks<W> sk{a};
   const uint32_t y = wid % N, x_id = wid / N * N;
   const size_t columns = a.waves_per_rank / N;
   const char *src = static_cast<const char *>(a.in.p[r]) + y * chunk;
@@ -485,9 +539,9 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
     // parallel_transmit.hpp:88-122), so the owner always finds its next messages
     // waiting and the column runs at the owner's pace.
     auto scatter = [&](size_t off, uint32_t step) {
-      const typename W::Reg p = W::load(src + off, bytes_left(chunk, off, W::kWireBytes), lane);
-      W::send(sk.scat(y, x_id + r, step % NSLOT), sk.sflag(y, x_id + r, step % NSLOT), p,
-              a.seq + step / NSLOT, lane);
+      const typename W::Reg p = W::load(src + off, bytes_left(chunk, off, W::kWireBytes), lane, nt);
+      const uint32_t slot = wl::parallel_slot(x_id, r, step % NSLOT);
+      W::send(sk.scat(y, slot), sk.sflag(y, slot), p, a.seq + step / NSLOT, lane);
     };
     for (uint32_t k = 0; k < kAhead; ++k)
       if (first + k * stride < chunk) scatter(first + k * stride, k);
@@ -497,8 +551,9 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
       const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
       if (off + kAhead * stride < chunk) scatter(off + kAhead * stride, t + kAhead);
       typename W::Reg v;
-      W::recv(sk.gath(r, x_id + y, s), sk.gflag(r, x_id + y, s), v, flag, lane, spin);
-      W::store(dst + off, left, lane, v);
+      const uint32_t slot = wl::parallel_slot(x_id, y, s);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+      W::store(dst + off, left, lane, v, nt);
     }
   } else {
     // Wait, reduce, broadcast.
@@ -506,24 +561,26 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
     for (size_t off = first; off < chunk; off += stride, ++t) {
       const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
       const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
-      typename W::Reg v = W::load(src + off, left, lane);
+      typename W::Reg v = W::load(src + off, left, lane, nt);
       const char *ms[N - 1];
       const uint32_t *mf[N - 1];
       typename W::Reg m[N - 1];
 #pragma unroll
       for (int i = 0; i < N - 1; ++i) {
         const int next = (r + i + 1) % N;
-        ms[i] = sk.scat(r, x_id + next, s);
-        mf[i] = sk.sflag(r, x_id + next, s);
+        const uint32_t slot = wl::parallel_slot(x_id, next, s);
+        ms[i] = sk.scat(r, slot);
+        mf[i] = sk.sflag(r, slot);
       }
       W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
       for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);    // peers in order rank+1, rank+2, ...
+      const uint32_t mine = wl::parallel_slot(x_id, r, s);
       for (int i = 0; i < N - 1; ++i) {
         const int next = (r + i + 1) % N;
-        W::send(sk.gath(next, x_id + r, s), sk.gflag(next, x_id + r, s), v, flag, lane);
+        W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
       }
-      W::store(dst + off, left, lane, v);
+      W::store(dst + off, left, lane, v, nt);
     }
   }
 }
@@ -532,9 +589,9 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
 // One wave does everything its rank owes a wire column, peer after peer.
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
-  constexpr int NSLOT = 4;
+  constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
-  const Sinks<W, NSLOT> sk{a};
+  const Sinks<W> sk{a};
   const uint32_t wpr = a.waves_per_rank;
   const char *src = static_cast<const char *>(a.in.p[r]);
   char *dst = static_cast<char *>(a.out.p[r]);
@@ -542,110 +599,108 @@ __global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
   for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
     const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    const uint32_t mine = wl::ring_slot(wpr, r, wid, s);
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      const typename W::Reg p = W::load(src + next * chunk + off, left, lane);
-      W::send(sk.scat(next, r * wpr + wid, s), sk.sflag(next, r * wpr + wid, s), p, flag, lane);
+      const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
+      W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
     }
-    typename W::Reg v = W::load(src + r * chunk + off, left, lane);
+    typename W::Reg v = W::load(src + r * chunk + off, left, lane, nt);
     const char *ms[N - 1];
     const uint32_t *mf[N - 1];
     typename W::Reg m[N - 1];
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      ms[i] = sk.scat(r, next * wpr + wid, s);
-      mf[i] = sk.sflag(r, next * wpr + wid, s);
+      const uint32_t slot = wl::ring_slot(wpr, (r + i + 1) % N, wid, s);
+      ms[i] = sk.scat(r, slot);
+      mf[i] = sk.sflag(r, slot);
     }
     W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);      // peers in order rank+1, rank+2, ...
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      W::send(sk.gath(next, r * wpr + wid, s), sk.gflag(next, r * wpr + wid, s), v, flag, lane);
+      W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
     }
-    W::store(dst + r * chunk + off, left, lane, v);
+    W::store(dst + r * chunk + off, left, lane, v, nt);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      ms[i] = sk.gath(r, next * wpr + wid, s);
-      mf[i] = sk.gflag(r, next * wpr + wid, s);
+      const uint32_t slot = wl::ring_slot(wpr, (r + i + 1) % N, wid, s);
+      ms[i] = sk.gath(r, slot);
+      mf[i] = sk.gflag(r, slot);
     }
     W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i)
-      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i]);
+      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i], nt);
   }
 }
 
 // ---- SimpleTransmit (simple_transmit.hpp:16-179) ---------------------------------------------
 // The older three-phase form: scatter / pollRecvReduceBcast / pollGatherOutputs.
 // Same data flow as the sequential transmit, but the sinks are linear rings: each
-// sender owns one 2 MiB section of every peer's sink, a message lands at
-// ringOffset = transmitted bytes % section, and the flag counts how often the
-// ring has wrapped (seqNo + transmitted bytes / section).
+// sender owns one section of every peer's sink, a message lands at ringOffset =
+// messages sent so far % section, and the flag counts how often the ring has
+// wrapped (seqNo + messages / section).  The host launches a power-of-two
+// number of wires per rank, so a ring position is only ever reused by the wave
+// that used it before.
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_simple(WireArgs a) {
-  constexpr uint32_t kSection = 0x200000;
-  constexpr uint32_t kPerSection = kSection / W::kSlotBytes;
+  constexpr uint32_t kPerSection = wl::kSimplePerSection;
   VR_WAVE_PROLOGUE;
+  const Sinks<W> sk{a};
   const uint32_t wpr = a.waves_per_rank;
   const char *src = static_cast<const char *>(a.in.p[r]);
   char *dst = static_cast<char *>(a.out.p[r]);
-  auto sink = [&](void *base, int section, uint32_t pos) {
-    return static_cast<char *>(base) + (size_t)section * kSection + (size_t)pos * W::kSlotBytes;
-  };
-  auto flagw = [&](void *base, int section, uint32_t pos) {
-    return static_cast<uint32_t *>(base) + (size_t)section * kPerSection + pos;
-  };
   size_t t = 0;
   for (size_t off = (size_t)wid * W::kWireBytes; off < chunk; off += (size_t)wpr * W::kWireBytes, ++t) {
     const size_t message = t * wpr + wid;                         // sinkOffset / wireTransSize
     const uint32_t pos = (uint32_t)(message % kPerSection);       // ringOffset
     const uint32_t flag = a.seq + (uint32_t)(message / kPerSection);   // seqNo + seqDelta
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
+    const uint32_t mine = wl::simple_slot(r, pos);
     for (int i = 0; i < N - 1; ++i) {                             // scatter
       const int next = (r + i + 1) % N;
-      const typename W::Reg p = W::load(src + next * chunk + off, left, lane);
-      W::send(sink(a.scatter.p[next], r, pos), flagw(a.sflag.p[next], r, pos), p, flag, lane);
+      const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
+      W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
     }
-    typename W::Reg v = W::load(src + r * chunk + off, left, lane);    // pollRecvReduceBcast
+    typename W::Reg v = W::load(src + r * chunk + off, left, lane, nt);    // pollRecvReduceBcast
     const char *ms[N - 1];
     const uint32_t *mf[N - 1];
     typename W::Reg m[N - 1];
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      ms[i] = sink(a.scatter.p[r], next, pos);
-      mf[i] = flagw(a.sflag.p[r], next, pos);
+      const uint32_t slot = wl::simple_slot((r + i + 1) % N, pos);
+      ms[i] = sk.scat(r, slot);
+      mf[i] = sk.sflag(r, slot);
     }
     W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);
-    W::store(dst + r * chunk + off, left, lane, v);               // write back locally first
+    W::store(dst + r * chunk + off, left, lane, v, nt);           // write back locally first
     for (int i = 0; i < N - 1; ++i) {
       const int next = (r + i + 1) % N;
-      W::send(sink(a.gather.p[next], r, pos), flagw(a.gflag.p[next], r, pos), v, flag, lane);
+      W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
     }
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) {                             // pollGatherOutputs
-      const int next = (r + i + 1) % N;
-      ms[i] = sink(a.gather.p[r], next, pos);
-      mf[i] = flagw(a.gflag.p[r], next, pos);
+      const uint32_t slot = wl::simple_slot((r + i + 1) % N, pos);
+      ms[i] = sk.gath(r, slot);
+      mf[i] = sk.gflag(r, slot);
     }
     W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i)
-      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i]);
+      W::store(dst + ((r + i + 1) % N) * chunk + off, left, lane, m[i], nt);
   }
 }
 
 // ---- RingTransmit::runAllreduce (sequential_transmit.hpp:429-472) ----------------------------
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
-  constexpr int NSLOT = 4;
+  constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
-  const Sinks<W, NSLOT> sk{a};
+  const Sinks<W> sk{a};
   const uint32_t wpr = a.waves_per_rank;
   const int next = (r + 1) % N;
   const char *src = static_cast<const char *>(a.in.p[r]);
@@ -655,34 +710,39 @@ __global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
     const uint32_t flag = a.seq + t / NSLOT, s = (a.seq + t) % NSLOT;
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
     int peer = r;
-    typename W::Reg v = W::load(src + peer * chunk + off, left, lane);           // step 0: send
-    W::send(sk.scat(next, peer * wpr + wid, s), sk.sflag(next, peer * wpr + wid, s), v, flag, lane);
+    uint32_t slot = wl::ring_slot(wpr, peer, wid, s);
+    typename W::Reg v = W::load(src + peer * chunk + off, left, lane, nt);       // step 0: send
+    W::send(sk.scat(next, slot), sk.sflag(next, slot), v, flag, lane);
     for (int i = 1; i < N - 1; ++i) {                                            // reduce and forward
       peer = (r + N - i) % N;
-      v = W::load(src + peer * chunk + off, left, lane);
+      slot = wl::ring_slot(wpr, peer, wid, s);
+      v = W::load(src + peer * chunk + off, left, lane, nt);
       typename W::Reg m;
-      W::recv(sk.scat(r, peer * wpr + wid, s), sk.sflag(r, peer * wpr + wid, s), m, flag, lane, spin);
+      W::recv(sk.scat(r, slot), sk.sflag(r, slot), m, flag, lane, spin);
       W::add(v, m);
-      W::send(sk.scat(next, peer * wpr + wid, s), sk.sflag(next, peer * wpr + wid, s), v, flag, lane);
+      W::send(sk.scat(next, slot), sk.sflag(next, slot), v, flag, lane);
     }
     peer = (r + 1) % N;                                                          // last add, start the gather ring
-    v = W::load(src + peer * chunk + off, left, lane);
+    slot = wl::ring_slot(wpr, peer, wid, s);
+    v = W::load(src + peer * chunk + off, left, lane, nt);
     {
       typename W::Reg m;
-      W::recv(sk.scat(r, peer * wpr + wid, s), sk.sflag(r, peer * wpr + wid, s), m, flag, lane, spin);
+      W::recv(sk.scat(r, slot), sk.sflag(r, slot), m, flag, lane, spin);
       W::add(v, m);
     }
-    W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
-    W::store(dst + peer * chunk + off, left, lane, v);
+    W::send(sk.gath(next, slot), sk.gflag(next, slot), v, flag, lane);
+    W::store(dst + peer * chunk + off, left, lane, v, nt);
     for (int i = 1; i < N - 1; ++i) {                                            // forward and write back
       peer = (r + 1 + N - i) % N;
-      W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
-      W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
-      W::store(dst + peer * chunk + off, left, lane, v);
+      slot = wl::ring_slot(wpr, peer, wid, s);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+      W::send(sk.gath(next, slot), sk.gflag(next, slot), v, flag, lane);
+      W::store(dst + peer * chunk + off, left, lane, v, nt);
     }
     peer = (r + 2) % N;                                                          // last hop: write back only
-    W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
-    W::store(dst + peer * chunk + off, left, lane, v);
+    slot = wl::ring_slot(wpr, peer, wid, s);
+    W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+    W::store(dst + peer * chunk + off, left, lane, v, nt);
   }
 }
 
@@ -690,9 +750,9 @@ __global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
 // chunk = bytes of one rank's slice; out[r] holds N slices.
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
-  constexpr int NSLOT = 4;
+  constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
-  const Sinks<W, NSLOT> sk{a};
+  const Sinks<W> sk{a};
   const uint32_t wpr = a.waves_per_rank;
   const int next = (r + 1) % N;
   const char *src = static_cast<const char *>(a.in.p[r]);
@@ -702,18 +762,21 @@ __global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
     const uint32_t flag = a.seq + t / NSLOT, s = (a.seq + t) % NSLOT;
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
     int peer = r;
-    typename W::Reg v = W::load(src + off, left, lane);
-    if (src != dst + (size_t)peer * chunk) W::store(dst + (size_t)peer * chunk + off, left, lane, v);
-    W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
+    uint32_t slot = wl::ring_slot(wpr, peer, wid, s);
+    typename W::Reg v = W::load(src + off, left, lane, nt);
+    if (src != dst + (size_t)peer * chunk) W::store(dst + (size_t)peer * chunk + off, left, lane, v, nt);
+    W::send(sk.gath(next, slot), sk.gflag(next, slot), v, flag, lane);
     for (int i = 1; i < N - 1; ++i) {
       peer = (r + N - i) % N;
-      W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
-      W::send(sk.gath(next, peer * wpr + wid, s), sk.gflag(next, peer * wpr + wid, s), v, flag, lane);
-      W::store(dst + (size_t)peer * chunk + off, left, lane, v);
+      slot = wl::ring_slot(wpr, peer, wid, s);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+      W::send(sk.gath(next, slot), sk.gflag(next, slot), v, flag, lane);
+      W::store(dst + (size_t)peer * chunk + off, left, lane, v, nt);
     }
     peer = (r + 1) % N;
-    W::recv(sk.gath(r, peer * wpr + wid, s), sk.gflag(r, peer * wpr + wid, s), v, flag, lane, spin);
-    W::store(dst + (size_t)peer * chunk + off, left, lane, v);
+    slot = wl::ring_slot(wpr, peer, wid, s);
+    W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+    W::store(dst + (size_t)peer * chunk + off, left, lane, v, nt);
   }
 }
 
@@ -723,12 +786,13 @@ __global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
 // of the same parity.
 template <int N, typename W>
 __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
-  constexpr int NSLOT = 8, B = N / 2;
+  constexpr uint32_t NSLOT = wl::kSlotsFlat;
+  constexpr int B = N / 2;
   VR_WAVE_PROLOGUE;
-  const Sinks<W, NSLOT> sk{a};
+  const Sinks<W> sk{a};
   const uint32_t y = wid % B, wg = wid / B * B;
-  const size_t columns = a.waves_per_rank / B;
-  const uint32_t far_base = a.waves_per_rank + B;     // the far sinks sit behind the close ones
+  const uint32_t wpr = a.waves_per_rank;
+  const size_t columns = wpr / B;
   const int h = r & 1, l = r >> 1, pair = r ^ 1;
   const size_t close_off = (h ? (size_t)B * chunk : 0) + y * chunk;
   const size_t far_off = (h ? 0 : (size_t)B * chunk) + y * chunk;
@@ -740,20 +804,22 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
   // and so uses one of its eight slots): scatterFar two steps ahead, the pair sum
   // and the close scatter one step ahead.  Same messages, slots and flag values.
   auto scatter_far = [&](size_t off, uint32_t step) {
-    const typename W::Reg f = W::load(src + far_off + off, bytes_left(chunk, off, W::kWireBytes), lane);
-    W::send(sk.scat(pair, far_base + wid, step % NSLOT), sk.sflag(pair, far_base + wid, step % NSLOT), f,
-            a.seq + step / NSLOT, lane);
+    const typename W::Reg f = W::load(src + far_off + off, bytes_left(chunk, off, W::kWireBytes), lane, nt);
+    const uint32_t slot = wl::bisect_far_slot(wpr, B, wid, step % NSLOT);
+    W::send(sk.scat(pair, slot), sk.sflag(pair, slot), f, a.seq + step / NSLOT, lane);
   };
   // Pair sum of a step, sent on to the chunk's owner unless this wave is the owner.
   auto pair_sum = [&](size_t off, uint32_t step) {
     const uint32_t s = step % NSLOT, flag = a.seq + step / NSLOT;
-    typename W::Reg v = W::load(src + close_off + off, bytes_left(chunk, off, W::kWireBytes), lane);
+    typename W::Reg v = W::load(src + close_off + off, bytes_left(chunk, off, W::kWireBytes), lane, nt);
     typename W::Reg m;
-    W::recv(sk.scat(r, far_base + wid, s), sk.sflag(r, far_base + wid, s), m, flag, lane, spin);
+    const uint32_t far = wl::bisect_far_slot(wpr, B, wid, s);
+    W::recv(sk.scat(r, far), sk.sflag(r, far), m, flag, lane, spin);
     W::add(v, m);
     if ((int)y != l) {
       const int owner = 2 * (int)y + h;
-      W::send(sk.scat(owner, wg + l, s), sk.sflag(owner, wg + l, s), v, flag, lane);
+      const uint32_t slot = wl::bisect_close_slot(wg, l, s);
+      W::send(sk.scat(owner, slot), sk.sflag(owner, slot), v, flag, lane);
     }
     return v;
   };
@@ -770,31 +836,34 @@ __global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
     if (off + stride < chunk) nxt = pair_sum(off + stride, t + 1);
     typename W::Reg v = cur;
     if ((int)y != l) {
-      W::recv(sk.gath(r, wg + y, s), sk.gflag(r, wg + y, s), v, flag, lane, spin);
+      const uint32_t slot = wl::bisect_close_slot(wg, y, s);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
     } else {
       const char *ms[B - 1];
       const uint32_t *mf[B - 1];
       typename W::Reg m[B - 1];
 #pragma unroll
       for (int i = 0; i < B - 1; ++i) {
-        const int l_next = (l + i + 1) % B;
-        ms[i] = sk.scat(r, wg + l_next, s);
-        mf[i] = sk.sflag(r, wg + l_next, s);
+        const uint32_t slot = wl::bisect_close_slot(wg, (l + i + 1) % B, s);
+        ms[i] = sk.scat(r, slot);
+        mf[i] = sk.sflag(r, slot);
       }
       W::template recv_many<B - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
       for (int i = 0; i < B - 1; ++i) W::add(v, m[i]);    // pair sums in order l+1, l+2, ...
+      const uint32_t mine = wl::bisect_close_slot(wg, l, s);
       for (int i = 0; i < B - 1; ++i) {
         const int nx = (r + i * 2 + 2) % N;
-        W::send(sk.gath(nx, wg + l, s), sk.gflag(nx, wg + l, s), v, flag, lane);
+        W::send(sk.gath(nx, mine), sk.gflag(nx, mine), v, flag, lane);
       }
     }
-    W::send(sk.gath(pair, far_base + wid, s), sk.gflag(pair, far_base + wid, s), v, flag, lane);
-    W::store(dst + close_off + off, left, lane, v);
+    const uint32_t far = wl::bisect_far_slot(wpr, B, wid, s);
+    W::send(sk.gath(pair, far), sk.gflag(pair, far), v, flag, lane);
+    W::store(dst + close_off + off, left, lane, v, nt);
     {                                                 // pollFarGatherOutput
       typename W::Reg m;
-      W::recv(sk.gath(r, far_base + wid, s), sk.gflag(r, far_base + wid, s), m, flag, lane, spin);
-      W::store(dst + far_off + off, left, lane, m);
+      W::recv(sk.gath(r, far), sk.gflag(r, far), m, flag, lane, spin);
+      W::store(dst + far_off + off, left, lane, m, nt);
     }
     cur = nxt;
   }
@@ -814,11 +883,16 @@ constexpr int kUnrollLL16 = 2;   // 1 KiB payload in a 2 KiB message
 constexpr int kUnrollLL64 = 4;   // 1920 B payload in a 2 KiB message
 constexpr int kUnrollFlag = 2;   // 2 KiB payload (16-byte lanes), flag word elsewhere
 
+static_assert(WireLL<kUnrollLL, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireLL16<kUnrollLL16, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireLL64<kUnrollLL64, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+
 // ---- host side --------------------------------------------------------------------------
 
 template <typename W>
 static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 grid, dim3 block,
-                              WireArgs &args, bool cooperative) {
+                              WireArgs &args, int cooperative, int cus) {
   void *kargs[] = {&args};
   const void *fn = nullptr;
 #define VR_PICK(NN)                                                                         \
@@ -843,11 +917,20 @@ static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 gri
   }
 #undef VR_PICK
   if (!fn) return hipErrorInvalidValue;
-  // Cooperative launch: the runtime refuses a grid that cannot be co-resident,
-  // which is what makes spinning on another work-group's progress safe.  The
-  // plain launch is for callers that accept "at most one work-group per CU on
-  // an otherwise idle device" as that guarantee and want the shorter launch path.
-  if (cooperative) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+  // Waves spin on other work-groups' progress, which is only safe when all of
+  // them are resident at once.  The occupancy query says how many work-groups of
+  // this kernel one compute unit holds; a grid within that bound is co-resident
+  // on a device that runs nothing else, and takes the plain launch path (about
+  // 16 us shorter).  A larger grid, or a caller who asks for it, goes through the
+  // cooperative launch, which makes the runtime check the same bound.
+  bool coop = cooperative == 1;
+  if (cooperative < 0) {
+    int per_cu = 0;
+    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, (int)block.x, 0);
+    if (e != hipSuccess) return e;
+    coop = (uint64_t)grid.x > (uint64_t)per_cu * (uint64_t)cus;
+  }
+  if (coop) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
   return hipLaunchKernel(fn, grid, block, kargs, 0, s);
 }
 
@@ -862,29 +945,28 @@ uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   }
 }
 
-uint32_t wire_slot_bytes_max() { return WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes; }
-
 template <int DT>
 static hipError_t launch_wire_dt(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves,
-                                 int nranks, dim3 grid, dim3 block, WireArgs &args, bool cooperative) {
+                                 int nranks, dim3 grid, dim3 block, WireArgs &args, int cooperative,
+                                 int cus) {
   if (fmt == WIRE_FMT_LL)
-    return launch_flow<WireLL<kUnrollLL, DT>>(s, flow, nranks, grid, block, args, cooperative);
+    return launch_flow<WireLL<kUnrollLL, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
   if (fmt == WIRE_FMT_LL64)
-    return launch_flow<WireLL64<kUnrollLL64, DT>>(s, flow, nranks, grid, block, args, cooperative);
+    return launch_flow<WireLL64<kUnrollLL64, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
   if (fmt == WIRE_FMT_LL16)
-    return launch_flow<WireLL16<kUnrollLL16, DT>>(s, flow, nranks, grid, block, args, cooperative);
+    return launch_flow<WireLL16<kUnrollLL16, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
   if (vec_halves == 8)
-    return launch_flow<WireFlag<kUnrollFlag, h8, DT>>(s, flow, nranks, grid, block, args, cooperative);
-  return launch_flow<WireFlag<kUnrollFlag, h4, DT>>(s, flow, nranks, grid, block, args, cooperative);
+    return launch_flow<WireFlag<kUnrollFlag, h8, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
+  return launch_flow<WireFlag<kUnrollFlag, h4, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
 }
 
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks_per_rank, uint32_t block_threads, WireArgs &args,
-                       bool cooperative, DType dtype) {
-  const dim3 grid(blocks_per_rank * nranks), block(block_threads);
+                       uint32_t blocks, uint32_t block_threads, WireArgs &args, int cooperative,
+                       int cus, DType dtype) {
+  const dim3 grid(blocks), block(block_threads);
   if (dtype == DT_BF16)
-    return launch_wire_dt<DT_BF16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative);
-  return launch_wire_dt<DT_F16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative);
+    return launch_wire_dt<DT_BF16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative, cus);
+  return launch_wire_dt<DT_F16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative, cus);
 }
 
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {

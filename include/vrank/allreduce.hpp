@@ -147,6 +147,16 @@ class VirtualRanks {
   int size() const { return nranks_; }
   void setTransport(int transport) { transport_ = transport; }
   int transport() const { return transport_; }
+  // Allocates the wire transport's scratch (main.cpp:241-251); idempotent.
+  void reserveWire() { check(vr_ctx_reserve_wire(ctx_)); }
+  // The C ABI never allocates inside a collective call: reserve the scratch before
+  // the first call that takes the wire transport (explicitly, or the default
+  // transport of `parallel`).
+  int transportFor(int algo) {
+    if (transport_ == VR_TRANSPORT_WIRE || (transport_ == VR_TRANSPORT_DEFAULT && algo == VR_ALGO_PARALLEL))
+      reserveWire();
+    return transport_;
+  }
   void setTuning(const char *key, int value) { check(vr_ctx_set_tuning(ctx_, key, value)); }
   void setDtype(int dtype) { check(vr_ctx_set_dtype(ctx_, dtype)); }
   // Waits for `stream` and reports a wire-transport poll time-out, if any.
@@ -194,20 +204,20 @@ struct AllReduce {
   // Enqueue on `stream`; in place on the constructor's buffers.
   void operator()(void *stream = nullptr) {
     ranks_.setDtype(dtype_of<T>::value);
-    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
   // "construct, then allreduce(stream, inputs, nelems)": run on other buffers of
   // a shape this object was built for.
   void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
     ranks_.setDtype(dtype_of<T>::value);
-    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                        &seqNo_));
   }
   void allreduce(void *stream, T *const inputs[], T *const outputs[], std::size_t nelems) {
     ranks_.setDtype(dtype_of<T>::value);
-    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)),
                        reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &seqNo_));
   }
@@ -256,12 +266,12 @@ struct bisectPAllReduce {
   }
   void operator()(void *stream = nullptr) {
     ranks_.setDtype(dtype_of<T>::value);
-    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(), bufs_, nullptr, nelems_,
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
   void allreduce(void *stream, T *const inputs[], std::size_t nelems) {
     ranks_.setDtype(dtype_of<T>::value);
-    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transport(),
+    check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo),
                        reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                        &seqNo_));
   }
@@ -305,7 +315,7 @@ struct AllGather {
     check(vr_check_allgather(algo, NRanks, ins_, outs_, nelems, &workSize_));
   }
   void operator()(void *stream = nullptr) {
-    check(vr_allgather(ranks_.get(), stream, algo, ranks_.transport(), ins_, outs_, nelems_, &seqNo_));
+    check(vr_allgather(ranks_.get(), stream, algo, ranks_.transportFor(algo), ins_, outs_, nelems_, &seqNo_));
   }
   static void launch(VirtualRanks &ranks, T *const inputs[], T *const outputs[], std::size_t nelems,
                      std::uint32_t &step, void *stream = nullptr) {
@@ -334,7 +344,7 @@ void testTransmit(const std::string &transmitType, LaunchParam launchParam, Virt
   check(vr_algo_from_string(transmitType.c_str(), &algo));
   if (vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
   ranks.setDtype(dtype_of<T>::value);
-  check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transport(),
+  check(vr_allreduce_grid(ranks.get(), stream, algo, ranks.transportFor(algo),
                           reinterpret_cast<void *const *>(const_cast<T **>(inputs)), nullptr, nelems,
                           step, launchParam.groups, launchParam.subgroups, launchParam.simd));
 }
@@ -347,7 +357,7 @@ void testAllgather(const std::string &transmitType, VirtualRanks &ranks, T *cons
   int algo = -1;
   check(vr_algo_from_string(transmitType.c_str(), &algo));
   if (!vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
-  check(vr_allgather(ranks.get(), stream, algo, ranks.transport(),
+  check(vr_allgather(ranks.get(), stream, algo, ranks.transportFor(algo),
                      reinterpret_cast<const void *const *>(const_cast<T **>(inputs)),
                      reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &step));
 }

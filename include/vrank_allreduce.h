@@ -20,9 +20,13 @@
  *   vr_algo_from_string<- the -a string switch                       allreduce.cpp:1128-1188, 1198-1212
  *   vr_fill_pattern   <- fill_pattern                                utils.hpp:15-19
  *   vr_parse_nelems   <- parse_nelems                                main.cpp:17-34
- *   vr_ctx_create     <- scratch allocation + zeroing + peer tables  main.cpp:224-283
- *                        (Level Zero IPC exchange, ipc_exchange.cpp, has no
- *                        counterpart: all virtual ranks live in one address space)
+ *   vr_ctx_create     <- per-process set-up                          main.cpp:212-227
+ *   vr_ctx_reserve_wire<- scratch allocation + zeroing + peer tables  main.cpp:241-283
+ *   vr_allreduce_rank <- AllReduce(input, nelems, rank, seqNo, scatterBuf, gatherBuf,
+ *                        peerBuf0[], peerBuf1[]) + queue.submit      allreduce.hpp:18-28, 64-74
+ *                        ParallelTransmit / BisectPTransmit ctors    parallel_transmit.hpp:36-60,
+ *                                                                    bisect_transmit.hpp:427-482
+ *   vr_rank_scratch_bytes <- interm_size = world * 8 MiB             main.cpp:241
  */
 #ifndef VRANK_ALLREDUCE_H
 #define VRANK_ALLREDUCE_H
@@ -103,12 +107,16 @@ typedef struct vr_ctx vr_ctx;
 
 /* ---- lifetime --------------------------------------------------------------- */
 
-/* Creates a context for `nranks` virtual ranks on HIP device `device`.  The
- * wire-transport scratch (per rank a scatter and a gather region plus flag words)
- * is allocated and zeroed once (main.cpp:241-251) by the first wire-transport
- * launch; the direct transport needs none.  nranks must be 2, 4, 8 or 16. */
+/* Creates a context for `nranks` virtual ranks on HIP device `device`.  nranks
+ * must be 2, 4, 8 or 16.  The direct transport needs no scratch. */
 int vr_ctx_create(int device, int nranks, vr_ctx **out);
 int vr_ctx_destroy(vr_ctx *ctx);
+/* Allocates and zeroes, once, the wire transport's scratch: one device allocation
+ * holding a scatter and a gather sink per rank (ipcbuf0 | ipcbuf1 and the peer
+ * tables of main.cpp:241-283).  This is the only place the wire transport
+ * allocates or synchronises: a wire-transport launch on a context whose scratch
+ * is not reserved returns VR_ERR_INVALID.  Idempotent. */
+int vr_ctx_reserve_wire(vr_ctx *ctx);
 int vr_ctx_nranks(const vr_ctx *ctx);
 int vr_ctx_set_dtype(vr_ctx *ctx, int dtype);   /* element type of the following collectives */
 int vr_ctx_get_dtype(const vr_ctx *ctx);
@@ -155,6 +163,28 @@ int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const
 int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void *const inputs[],
                  void *const outputs[], size_t nelems, uint32_t *seq_no);
 
+/* One rank of a wire-transport all-reduce against caller-owned scratch: the form
+ * the reference constructs in every process.  The launch holds `rank`'s wires
+ * only; the other ranks' launches (other streams of this process, or other
+ * processes that mapped the same sinks) must run at the same time, since every
+ * wave waits, with a bounded spin, for its peers' messages.
+ *   input / output : this rank's buffer (output NULL = in place).
+ *   scatter_buf, gather_buf : this rank's own sinks; peer_buf0[q] / peer_buf1[q]
+ *              the scatter / gather sink of rank q (entry `rank` is ignored).
+ *              Each sink holds `sink_bytes` >= vr_rank_scratch_bytes() bytes, is
+ *              16-byte aligned, and was zeroed once before the first launch.
+ *   seq_no   : in/out; must be the same on every rank and only ever grow; a
+ *              change of algo needs freshly zeroed sinks.
+ * Same validation and error codes as vr_allreduce for this rank's pointers.  The
+ * library neither allocates nor clears anything here.  vr_ctx_check(ctx, stream)
+ * reports a time-out of this context's launches. */
+int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
+                      void *scatter_buf, void *gather_buf, void *const peer_buf0[],
+                      void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+/* Bytes a scatter sink (and equally a gather sink) must hold for this context's
+ * rank count, device and "wire_blocks_per_cu" setting. */
+int vr_rank_scratch_bytes(const vr_ctx *ctx, size_t *sink_bytes);
+
 /* Reference test-harness flavour (testTransmit with a user grid, main.cpp:289-314):
  * `groups` x `subgroups` sub-groups of `simd` lanes.  Results never depend on the
  * grid; unusable grids are rejected the way the reference's host code rejects
@@ -181,12 +211,15 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * for the wire transport "wire_fenced" (1 = the Rt64_128 family sends payload
  * lines with a separate flag word ordered by agent-scope release/acquire fences
  * instead of 64-byte segments with an embedded flag) and
- * "wire_cooperative" (0 = plain launch instead of a cooperative one),
+ * "wire_cooperative" (0 = plain launch, 1 = cooperative launch; by default a plain
+ * launch whenever the occupancy query proves the grid co-resident),
+ * "wire_stream_io" (1 = inputs loaded and outputs stored with streaming cache
+ * policies; default 0 = cached, which measured faster at every size),
  * "wire_ahead" (1..6 steps the parallel flow's scatters run ahead of its gathers),
  * "wire_msg16" (0 = the Rt64_PCIE family sends self-validating 8-byte messages
  * instead of 16-byte stores that carry the flag twice) and
- * "wire_blocks_per_cu" (1..4 resident work-groups per CU; set it before the first
- * wire-transport launch, it sizes the scratch).
+ * "wire_blocks_per_cu" (1..4 resident work-groups per CU; set it before
+ * vr_ctx_reserve_wire, it sizes the scratch).
  * -1 restores the library's own choice. */
 int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value);
 int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);

@@ -17,7 +17,8 @@ def pytest_configure(config):
              os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main"),
              os.path.join(ROOT, "oracle", "libvr_oracle.so"),
              os.path.join(ROOT, "tests", "cpp", "test_host_api"),
-             os.path.join(ROOT, "tests", "cpp", "test_graph")]
+             os.path.join(ROOT, "tests", "cpp", "test_graph"),
+             os.path.join(ROOT, "tests", "cpp", "test_wire_layout")]
     if not all(os.path.exists(p) for p in built):
         import __graft_entry__
         __graft_entry__.build()

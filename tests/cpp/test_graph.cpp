@@ -108,6 +108,26 @@ int main() {
   HIPCK(hipEventElapsedTime(&ms_eager, e0, e1));
   printf("10-kernel sequence: graph replay %.1f us, eager %.1f us\n", ms_graph * 1e3 / 50, ms_eager * 1e3 / 50);
 
+  // The wire transport refuses capture: its flag values are per-launch kernel
+  // arguments, so a replay would read stale flags.
+  {
+    int parallel_id = -1;
+    VRCK(vr_algo_from_string("parallel", &parallel_id));
+    VRCK(vr_ctx_reserve_wire(ctx));
+    hipGraph_t g2;
+    HIPCK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    const int rc = vr_allreduce(ctx, stream, parallel_id, VR_TRANSPORT_WIRE, in, mid, n, &seq);
+    HIPCK(hipStreamEndCapture(stream, &g2));
+    (void)hipGraphDestroy(g2);
+    if (rc != VR_ERR_INVALID) {
+      printf("wire launch under capture returned %d, expected VR_ERR_INVALID\n", rc);
+      ++failures;
+    }
+    // and works again outside capture
+    VRCK(vr_allreduce(ctx, stream, parallel_id, VR_TRANSPORT_WIRE, in, mid, n, &seq));
+    VRCK(vr_ctx_check(ctx, stream));
+  }
+
   (void)hipGraphExecDestroy(exec);
   (void)hipGraphDestroy(graph);
   for (int r = 0; r < N; ++r) {

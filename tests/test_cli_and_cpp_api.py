@@ -13,6 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
 CPP_TEST = os.path.join(ROOT, "tests", "cpp", "test_host_api")
 GRAPH_TEST = os.path.join(ROOT, "tests", "cpp", "test_graph")
+LAYOUT_TEST = os.path.join(ROOT, "tests", "cpp", "test_wire_layout")
 
 
 def run(cmd, **kw):
@@ -22,6 +23,13 @@ def run(cmd, **kw):
 def test_cli_and_cpp_test_are_built():
     assert os.path.exists(CLI), "run __graft_entry__.build()"
     assert os.path.exists(CPP_TEST), "run make -C tests/cpp"
+
+
+def test_wire_sinks_hold_every_slot_the_kernels_index():
+    """CPU walk over every flow x rank count x wire count with the kernels' own
+    slot functions: each message slot and flag word lies inside the sink."""
+    r = run([LAYOUT_TEST], timeout=120)
+    assert r.returncode == 0 and " 0 failures" in r.stdout, r.stdout
 
 
 def test_cli_rejects_bad_arguments_like_the_reference():

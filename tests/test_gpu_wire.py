@@ -225,7 +225,7 @@ def test_allgather_wire(ctxs, oracle, nranks, algo):
 
 
 @pytest.mark.parametrize("algo", ["simple", "parallel", "bisect", "simple_ring", "simple_pcie",
-                                  "simple_pcie_p"])
+                                  "simple_pcie_p", "simple_transmit"])
 def test_fenced_flag_word_format(oracle, algo):
     """The Rt64_128 family can also travel as payload lines + a separate flag word
     ordered by agent-scope release/acquire fences (no store-atomicity assumption)."""
@@ -240,13 +240,58 @@ def test_fenced_flag_word_format(oracle, algo):
     ctx.close()
 
 
-def test_plain_launch_instead_of_cooperative(oracle):
+@pytest.mark.parametrize("cooperative", [0, 1])
+def test_plain_and_cooperative_launch(oracle, cooperative):
+    """By default the launch is plain when the occupancy query proves the grid
+    co-resident; both forms can be forced."""
     ctx = vr.VirtualRanks(8)
-    ctx.set_tuning(wire_cooperative=0)
+    ctx.set_tuning(wire_cooperative=cooperative)
     for algo in ("small", "simple", "bisect", "small_ring"):
         ins = H.make_inputs(oracle, 8, 1 << 18, 6100)
         got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE)
         H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), algo)
+    ctx.close()
+
+
+def test_collective_calls_never_allocate_the_scratch(oracle):
+    """The C ABI allocates the wire transport's scratch in vr_ctx_reserve_wire only:
+    a wire launch on an unreserved context is an error, not a hidden hipMalloc."""
+    import ctypes as C
+    from gpu_ipc_example_amd import binding
+    L = vr.lib()
+    h = C.c_void_p()
+    assert L.vr_ctx_create(0, 8, C.byref(h)) == 0
+    n = 8 * 4096
+    ins = H.make_inputs(oracle, 8, n, 6150)
+    src = H.RankBuffers(8, n)
+    src.upload(ins)
+    seq = C.c_uint32(1)
+    table = binding._table(src.ptrs)
+    for algo, transport in (("parallel", vr.TRANSPORT_DEFAULT), ("simple", WIRE)):
+        rc = L.vr_allreduce(h, None, vr.algo_id(algo), transport, table, None, n, C.byref(seq))
+        assert rc == 7 and b"vr_ctx_reserve_wire" in L.vr_last_error_detail()
+    assert L.vr_ctx_reserve_wire(h) == 0 and L.vr_ctx_reserve_wire(h) == 0
+    assert L.vr_allreduce(h, None, vr.algo_id("parallel"), vr.TRANSPORT_DEFAULT, table, None, n,
+                          C.byref(seq)) == 0
+    assert L.vr_ctx_check(h, None) == 0
+    H.assert_all_ranks_equal(oracle, src.download(), oracle.rotated(ins))
+    src.free()
+    L.vr_ctx_destroy(h)
+
+
+@pytest.mark.parametrize("stream_io", [0, 1])
+def test_streaming_and_cached_io(oracle, stream_io):
+    """Inputs and outputs move with cached or with streaming accesses; ragged
+    tails go through the same bounds-checked buffer accesses either way."""
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_stream_io=stream_io)
+    for algo in ("small", "parallel", "bisect", "small_ring", "simple_pcie", "simple_transmit"):
+        for n in (64 * 1, 64 * 1001, 1 << 19):
+            for inplace in (True, False):
+                ins = H.make_inputs(oracle, 8, n, 6160 + n)
+                got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, inplace=inplace)
+                H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins),
+                                         "%s n=%d io=%d" % (algo, n, stream_io))
     ctx.close()
 
 
