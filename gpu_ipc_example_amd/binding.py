@@ -71,6 +71,7 @@ def lib():
         "vr_ctx_nranks": (i, [vp]),
         "vr_allreduce_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
         "vr_rank_scratch_bytes": (i, [vp, C.POINTER(sz)]),
+        "vr_allreduce_static": (i, [vp, vp, i, vpp, vpp, sz]),
         "vr_ctx_set_dtype": (i, [vp, i]),
         "vr_ctx_get_dtype": (i, [vp]),
         "vr_fill_pattern_dt": (None, [i, C.POINTER(C.c_uint16), i, sz]),
@@ -270,6 +271,23 @@ class VirtualRanks:
                                        _table(peers0), _table(peers1), sink_bytes, nelems,
                                        C.byref(seq)))
         return seq.value
+
+    def allreduce_static(self, algo, bufs, nelems, outs=None, stream=None):
+        """Wire-transport all-reduce through the library's fixed scratch region (no allocation)."""
+        _check(lib().vr_allreduce_static(self._h, stream, algo_id(algo), _table(bufs),
+                                         _table(outs) if outs is not None else None, nelems))
+
+    def set_tuning(self, **kw):
+        for k, v in kw.items():
+            _check(lib().vr_ctx_set_tuning(self._h, k.encode(), int(v)))
+
+    def get_tuning(self, key):
+        v = C.c_int(0)
+        _check(lib().vr_ctx_get_tuning(self._h, key.encode(), C.byref(v)))
+        return v.value
+
+    def set_spin_limit(self, polls):
+        _check(lib().vr_ctx_set_spin_limit(self._h, polls))
 
     def allreduce(self, algo, bufs, nelems, outs=None, transport=TRANSPORT_DEFAULT, stream=None):
         assert len(bufs) == self.nranks

@@ -263,6 +263,7 @@ struct vr_ctx {
   DType dtype = DT_F16;
   uint32_t *status = nullptr;     // time-out word of this context's wire launches (256 B)
   WireState wire;
+  bool static_used = false;       // vr_allreduce_static has run on this context
 };
 
 static const uint32_t kDefaultSpinLimit = 1u << 22;
@@ -467,6 +468,22 @@ static int wire_launch_ctx(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const Pt
 }
 
 
+// The library's fixed scratch region on the context's device: its sinks (for the
+// context's rank count) and its status word.
+static int static_sinks(const vr_ctx *ctx, WireSinks *k, uint32_t **status) {
+  void *fixed = nullptr;
+  size_t bytes = 0;
+  hipError_t e = wire_static_scratch(ctx->dev.device, &fixed, &bytes);
+  if (e != hipSuccess) return fail_hip(e, "hipGetSymbolAddress(scratch)");
+  const wl::Layout l = wl::layout_for(ctx->nranks, kStaticWiresPerRank, false);
+  if ((size_t)ctx->nranks * l.rank_bytes + 256 > bytes)
+    return fail(VR_ERR_INVALID, "the fixed scratch region holds at most " +
+                                    std::to_string(kStaticMaxRanks) + " ranks");
+  sinks_at(k, ctx->nranks, static_cast<char *>(fixed), l, kStaticWiresPerRank, false);
+  *status = reinterpret_cast<uint32_t *>(static_cast<char *>(fixed) + bytes - 256);
+  return VR_OK;
+}
+
 extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   if (!out) return fail(VR_ERR_INVALID, "null out");
   *out = nullptr;
@@ -483,10 +500,14 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(VR_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", kernels are built for gfx950");
   HIP_TRY(hipSetDevice(device));
-  // Set-up work that must not happen in a hot call: the context's time-out word.
+  // Set-up work that must not happen in a hot call: the context's time-out word,
+  // and the device address of the library's fixed scratch region on this device.
   uint32_t *status = nullptr;
   HIP_TRY(hipMalloc((void **)&status, 256));
   hipError_t e = hipMemset(status, 0, 256);
+  void *fixed = nullptr;
+  size_t fixed_bytes = 0;
+  if (e == hipSuccess) e = wire_static_scratch(device, &fixed, &fixed_bytes);
   if (e != hipSuccess) {
     (void)hipFree(status);
     return fail_hip(e, "vr_ctx_create set-up");
@@ -783,6 +804,36 @@ extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transp
                        wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &next);
 }
 
+// Largest input the allocation-free entry point accepts: the sweep's largest
+// point, 256 MiB per rank.
+static const size_t kStaticMaxBytesPerRank = 256ull << 20;
+
+extern "C" int vr_allreduce_static(vr_ctx *ctx, void *stream, int algo, void *const bufs[],
+                                   void *const outs[], size_t nelems) {
+  Prepared p;
+  if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
+  if (ctx->nranks > kStaticMaxRanks)
+    return fail(VR_ERR_INVALID, "vr_allreduce_static serves at most " + std::to_string(kStaticMaxRanks) +
+                                    " ranks, this context has " + std::to_string(ctx->nranks));
+  if (nelems * 2 > kStaticMaxBytesPerRank)
+    return fail(VR_ERR_INVALID, "vr_allreduce_static serves at most " +
+                                    std::to_string(kStaticMaxBytesPerRank) + " bytes per rank, got " +
+                                    std::to_string(nelems * 2));
+  if (p.a->wire_flow() == WIRE_SIMPLE)
+    return fail(VR_ERR_INVALID, "vr_allreduce_static has no room for SimpleTransmit's 2 MiB sender sections");
+  WireSinks k;
+  uint32_t *status = nullptr;
+  if (int rc = static_sinks(ctx, &k, &status)) return rc;
+  // The region is shared by every context on the device and keeps the last
+  // call's messages: every call clears the sinks first (a fill kernel on the
+  // stream), so the flags can start from 1 each time.
+  const WireLaunch wlch = {&k, nullptr, status, -1, true};
+  uint32_t seq = 1, used = 0;
+  ctx->static_used = true;
+  return wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, &seq,
+                     0, &used, wlch);
+}
+
 // One rank of an all-reduce, the form the reference constructs per process
 // (allreduce.hpp:18-28, parallel_transmit.hpp:36-60, bisect_transmit.hpp:427-482).
 extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
@@ -935,6 +986,12 @@ extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
     if (int rc = wire_clear(ctx->wire.sinks, ctx->nranks, (hipStream_t)stream)) return rc;
     ctx->wire.hist.used = false;
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  }
+  if (ctx->static_used) {
+    WireSinks k;
+    uint32_t *word = nullptr;
+    if (int rc = static_sinks(ctx, &k, &word)) return rc;
+    if (int rc = check_status_word(word, &timed_out)) return rc;   // its sinks are cleared by every call
   }
   if (timed_out)
     return fail(VR_ERR_TIMEOUT, "a wire-transport poll exceeded the spin limit; scratch was reset");

@@ -98,6 +98,11 @@ hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_hal
                        uint32_t blocks, uint32_t block_threads, WireArgs &args,
                        int cooperative, int cus, DType dtype);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
+// The library's own fixed scratch region in device memory (one per GPU, held
+// until the process ends): its device address on the current device and its size.
+constexpr uint32_t kStaticWiresPerRank = 32;
+constexpr int kStaticMaxRanks = 8;
+hipError_t wire_static_scratch(int device, void **ptr, size_t *bytes);
 
 
 #ifdef __HIPCC__

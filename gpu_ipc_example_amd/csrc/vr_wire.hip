@@ -888,6 +888,34 @@ static_assert(WireLL16<kUnrollLL16, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "s
 static_assert(WireLL64<kUnrollLL64, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 static_assert(WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 
+// ---- the library's own scratch -----------------------------------------------------------
+// Fixed region for the entry point that must not allocate: every rank's scatter
+// and gather sink for up to kStaticMaxRanks ranks of kStaticWiresPerRank wires
+// (no SimpleTransmit sections), then 256 bytes that hold the status word.  In
+// host code the array's name is only a handle: its device address is looked up
+// once per device with hipGetSymbolAddress.
+constexpr size_t kStaticScratchBytes =
+    (size_t)kStaticMaxRanks * wl::layout_for(kStaticMaxRanks, kStaticWiresPerRank, false).rank_bytes + 256;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_static_ptr[kMaxDevices];
+
+hipError_t wire_static_scratch(int device, void **ptr, size_t *bytes) {
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  if (!g_static_ptr[device]) {
+    // The caller has made `device` current: each GPU holds its own copy of the
+    // array at its own address.
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_static_ptr[device] = p;
+  }
+  *ptr = g_static_ptr[device];
+  *bytes = kStaticScratchBytes;
+  return hipSuccess;
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 template <typename W>

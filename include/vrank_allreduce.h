@@ -185,6 +185,21 @@ int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input
  * rank count, device and "wire_blocks_per_cu" setting. */
 int vr_rank_scratch_bytes(const vr_ctx *ctx, size_t *sink_bytes);
 
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  A wire-transport vr_allreduce whose sinks live in a fixed
+ * region of device memory that is part of the library's code object (about
+ * 32 MiB per GPU, held until the process ends) instead of scratch reserved by the
+ * context.  Calls no hipMalloc / hipFree and does not synchronise.
+ * Limits: at most 8 ranks, at most 256 MiB (134217728 elements) per rank, every
+ * all-reduce algo except simple_transmit; 32 wires per rank.  Beyond them:
+ * VR_ERR_INVALID.  Every context on a GPU shares that GPU's region and each call
+ * clears it first (on `stream`), so calls that overlap in time on one GPU race:
+ * keep them on one stream or otherwise ordered.  Time-outs are reported by
+ * vr_ctx_check like those of vr_allreduce. */
+int vr_allreduce_static(vr_ctx *ctx, void *stream, int algo, void *const bufs[], void *const outs[],
+                        size_t nelems);
+
 /* Reference test-harness flavour (testTransmit with a user grid, main.cpp:289-314):
  * `groups` x `subgroups` sub-groups of `simd` lanes.  Results never depend on the
  * grid; unusable grids are rejected the way the reference's host code rejects
