@@ -45,7 +45,12 @@ WORKLOADS = {
     "cfg4": (4, "allgather_simple", 4194304, 0, -2.0, 2.0, 4000),
     # the 16-rank instantiation of bisect (allreduce.cpp:1020), same 256 MiB of inputs as cfg3
     "bisect16": (16, "bisect", 8388608, 1, 0.0, 0.02, 6000),
+    # one point of the size sweep: its named protocol (message passing) at 32 MiB per rank
+    "cfg5_32MiB": (8, "parallel", 16777216, 1, 0.0, 1.0, 5000),
 }
+
+# --transport: how the virtual ranks exchange data (0 = the protocol's default).
+TRANSPORT = 0
 
 
 def describe(name):
@@ -89,9 +94,10 @@ def setup(vr, binding, name, inplace, nsets=1):
 def launch(ctx, name, ins, outs):
     n, algo, ne, *_ = WORKLOADS[name]
     if algo.startswith("allgather"):
-        ctx.allgather(algo, [b.ptr for b in ins], [b.ptr for b in outs], ne)
+        ctx.allgather(algo, [b.ptr for b in ins], [b.ptr for b in outs], ne, transport=TRANSPORT)
     else:
-        ctx.allreduce(algo, [b.ptr for b in ins], ne, outs=[b.ptr for b in outs] if outs else None)
+        ctx.allreduce(algo, [b.ptr for b in ins], ne, outs=[b.ptr for b in outs] if outs else None,
+                      transport=TRANSPORT)
 
 
 def time_kernels(binding, ctx, name, sets, iters, group=1):
@@ -254,6 +260,9 @@ def main():
                          "known-size kernel that hardware-counter readings are scaled by")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"],
                     help="element type of the adds (the reference instantiates both)")
+    ap.add_argument("--transport", default="default", choices=["default", "direct", "wire"],
+                    help="direct: one pass over HBM; wire: the reference's message passing through "
+                         "scratch; default: wire for 'parallel', direct otherwise")
     ap.add_argument("--inplace", action="store_true",
                     help="reference semantics: results overwrite the inputs (values saturate "
                          "after a few steps; traffic is identical)")
@@ -281,8 +290,10 @@ def main():
     import gpu_ipc_example_amd as vr
     from gpu_ipc_example_amd import binding
 
-    global DTYPE
+    global DTYPE, TRANSPORT
     DTYPE = 1 if args.dtype == "bf16" else 0
+    TRANSPORT = {"default": vr.TRANSPORT_DEFAULT, "direct": vr.TRANSPORT_DIRECT,
+                 "wire": vr.TRANSPORT_WIRE}[args.transport]
 
     if args.sweep:
         sweep(vr, binding, args)
@@ -334,6 +345,7 @@ def main():
         launch(ctx, name, *sets[i % len(sets)])
     ctx.sync()
     wall = time.perf_counter() - t0
+    ctx.check()            # outside the timed region: a wire-transport poll time-out voids the run
     ms_per_step = wall / args.steps * 1e3
     value = B / (wall / args.steps) / 1e9
 
@@ -350,6 +362,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": DTYPE_NAMES[DTYPE], "data": "synthetic",
         "config": {"workload": describe(name), "virtual_ranks": n, "protocol": algo,
+                   "transport": args.transport,
                    "bytes_per_rank": ne * 2, "in_place": bool(args.inplace),
                    "algorithmic_bytes_per_step": B, "buffer_sets_rotated": len(sets),
                    "note": "steps rotate through %d buffer sets (%.0f MiB touched) so the 256 MiB "

@@ -347,6 +347,23 @@ class VirtualRanks:
         return np.frombuffer(ms, np.float32).copy()
 
 
+class Stream:
+    """A non-blocking HIP stream (vr_stream_create); `.handle` is the hipStream_t."""
+
+    def __init__(self, device=0):
+        h = C.c_void_p()
+        _check(lib().vr_stream_create(device, C.byref(h)))
+        self.handle = h
+
+    def sync(self):
+        _check(lib().vr_stream_sync(self.handle))
+
+    def close(self):
+        if self.handle:
+            lib().vr_stream_destroy(self.handle)
+            self.handle = None
+
+
 class EventTimer:
     """Pairs of HIP events recorded on one stream around caller-chosen launches."""
 

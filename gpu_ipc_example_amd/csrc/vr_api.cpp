@@ -80,9 +80,11 @@ struct AlgoInfo {
     }
   }
   // Rt64 -> self-validating 8-byte messages; Rt64_PCIE -> 16-byte messages with
-  // the flag twice; Rt64_128 family -> 64-byte segments of 15 payload dwords and a flag.
+  // the flag twice; Rt64_128 -> 128-byte messages, Rt64_128_PCIE -> 256-byte
+  // messages, both with a flag in every 64 bytes.
   WireFormat wire_format() const {
-    return !latency_tuned ? WIRE_FMT_LL64 : msg_bytes == 16 ? WIRE_FMT_LL16 : WIRE_FMT_LL;
+    if (latency_tuned) return msg_bytes == 16 ? WIRE_FMT_LL16 : WIRE_FMT_LL;
+    return msg_bytes == 16 ? WIRE_FMT_RT256 : WIRE_FMT_RT128;
   }
 };
 
@@ -267,7 +269,7 @@ struct vr_ctx {
 };
 
 static const uint32_t kDefaultSpinLimit = 1u << 22;
-static const int kWireBlocksPerCu = 2;
+static const int kWireBlocksPerCu = 3;
 static const uint32_t kWireAhead = 4;
 
 static void wire_free(vr_ctx *c) {
@@ -357,7 +359,11 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const int N = c->nranks;
   const WireFlow flow = a->wire_flow();
   WireFormat fmt = a->wire_format();
-  if (fmt == WIRE_FMT_LL64 && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
+  const bool big = fmt == WIRE_FMT_RT128 || fmt == WIRE_FMT_RT256;
+  if (big && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
+  // Self-validating 8-byte messages for the Rt64_128 families too: nothing beyond
+  // 8-byte store atomicity is assumed, at half the payload per message.
+  if (big && c->tune.wire_fenced == 2) fmt = WIRE_FMT_LL;
   if (fmt == WIRE_FMT_LL16 && c->tune.wire_msg16 == 0) fmt = WIRE_FMT_LL;
   if (flow == WIRE_SIMPLE && !k.simple_ok)
     return fail(VR_ERR_INVALID, "these sinks have no room for SimpleTransmit's 2 MiB sender sections");
@@ -371,10 +377,22 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
                                   "are per-launch kernel arguments (capture the direct transport)");
     (void)hipGetLastError();
   }
+  // `parallel` names the transmit, not a wire format: it takes the reference's
+  // 256-byte messages (16 bytes per lane) when every pointer and the chunk allow
+  // 16-byte accesses, its 128-byte messages otherwise.
+  if (fmt == WIRE_FMT_RT128 && a == &kAlgos[VR_ALGO_PARALLEL] && vec_halves == 8 && chunk_bytes % 16 == 0)
+    fmt = WIRE_FMT_RT256;
   const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
   const uint32_t waves_per_block = kWireBlockThreads / 64;
-  const uint32_t wpr_limit = k.wpr_max / psg * psg;
-  if (wpr_limit < psg) return fail(VR_ERR_INVALID, "sinks too small for this rank count");
+  // Every wave may wait for any other: keep the grid (for one-rank launches: the N
+  // grids together) within what the device holds at once.
+  int per_cu = 0;
+  if (hipError_t e = wire_blocks_per_cu(flow, fmt, vec_halves, N, kWireBlockThreads, c->dtype, &per_cu))
+    return fail_hip(e, "occupancy query");
+  const uint32_t resident_wpr = (uint32_t)((size_t)c->dev.cus * (size_t)per_cu / (size_t)N) * waves_per_block;
+  const uint32_t wpr_cap = k.wpr_max < resident_wpr ? k.wpr_max : resident_wpr;
+  const uint32_t wpr_limit = wpr_cap / psg * psg;
+  if (wpr_limit < psg) return fail(VR_ERR_INVALID, "sinks or device too small for this rank count");
   const uint32_t wire_bytes = wire_bytes_per_step(fmt, vec_halves);
   const size_t wires_per_chunk = div_up(chunk_bytes, wire_bytes);
   if (wires_per_chunk == 0) { *flags_used = 0; return VR_OK; }
@@ -436,16 +454,20 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   args.status = wlch.status;
   args.ahead = c->tune.wire_ahead > 0 ? (uint32_t)c->tune.wire_ahead : kWireAhead;
   args.solo_rank = wlch.solo_rank;
-  // Cached accesses measured faster than streaming ones for the wires' narrow
-  // per-lane inputs and outputs (a write-through store of part of a line costs a
-  // read-modify-write at the memory side); streaming stays selectable.
-  args.stream_io = c->tune.wire_stream_io > 0 ? 1u : 0u;
+  // Inputs and outputs that cannot stay in the 256 MiB memory-side cache anyway are
+  // streamed past it, which leaves that cache to the sinks (measured: faster from
+  // 256 MiB of inputs + outputs on, slower below).
+  const size_t io_bytes = 2 * (size_t)N * chunk_bytes * (a->allgather ? 1 : (size_t)N);
+  args.stream_io = c->tune.wire_stream_io >= 0 ? (uint32_t)c->tune.wire_stream_io
+                                               : (io_bytes >= (256ull << 20) ? 1u : 0u);
   const bool solo = wlch.solo_rank >= 0;
-  // One rank's launch cannot vouch for the other ranks' work-groups: plain launch.
-  const int cooperative = solo ? 0 : c->tune.wire_cooperative;
+  // The grid is co-resident by construction; a cooperative launch (on request)
+  // lets the runtime check that once more.  One rank's launch cannot vouch for
+  // the other ranks' work-groups: always plain.
+  const bool cooperative = !solo && c->tune.wire_cooperative == 1;
   const uint32_t blocks = solo ? blocks_per_rank : blocks_per_rank * (uint32_t)N;
   hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks, kWireBlockThreads, args,
-                             cooperative, c->dev.cus, c->dtype);
+                             cooperative, c->dtype);
   if (e != hipSuccess) return fail_hip(e, "launch_wire");
   if (wlch.hist) {
     wlch.hist->used = true;
@@ -576,10 +598,12 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "waves_per_cu must be in [1,64]");
     if (!strcmp(key, "unroll") && !(value == 1 || value == 2 || value == 4))
       return fail(VR_ERR_INVALID, "unroll must be 1, 2 or 4");
-    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_fenced") || !strcmp(key, "wire_msg16") || !strcmp(key, "f16_wide") || !strcmp(key, "wire_stream_io") ||
+    if ((!strcmp(key, "nt_load") || !strcmp(key, "oneshot") || !strcmp(key, "wire_msg16") || !strcmp(key, "f16_wide") || !strcmp(key, "wire_stream_io") ||
          !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
+    if (!strcmp(key, "wire_fenced") && (value < 0 || value > 2))
+      return fail(VR_ERR_INVALID, "wire_fenced must be 0 (embedded flags), 1 (flag words with fences), 2 (8-byte messages) or -1");
     if (!strcmp(key, "nt_store") && (value < 0 || value > 2))
       return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
     if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))

@@ -70,9 +70,10 @@ hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device
 enum WireFlow : int { WIRE_PARALLEL, WIRE_SEQUENTIAL, WIRE_RING, WIRE_BISECT, WIRE_ALLGATHER, WIRE_SIMPLE };
 enum WireFormat : int {
   WIRE_FMT_LL = 0,    // 4 B payload + 4 B flag per 8-byte store (Rt64 family)
-  WIRE_FMT_LL64 = 1,  // 60 B payload + 4 B flag per 64-byte segment (Rt64_128 family)
+  WIRE_FMT_RT128 = 1, // the reference's 128-byte message: 120 B payload, a flag per 64-byte half (Rt64_128)
   WIRE_FMT_FLAG = 2,  // 16 B payload lines + one fenced flag word per message
   WIRE_FMT_LL16 = 3,  // 8 B payload + the flag twice per 16-byte store (Rt64_PCIE family)
+  WIRE_FMT_RT256 = 4, // the reference's 256-byte message: 240 B payload, a flag per 64 bytes (Rt64_128_PCIE)
 };
 constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
 
@@ -91,12 +92,13 @@ struct WireArgs {
 };
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves);
-// Chooses a plain launch when the occupancy query proves that `blocks` work-groups
-// of the flow's kernel are co-resident on `cus` compute units, a cooperative
-// launch otherwise.  cooperative: -1 automatic, 0 plain, 1 cooperative.
+// Work-groups of the flow's kernel one compute unit holds at once (occupancy query).
+hipError_t wire_blocks_per_cu(WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
+                              uint32_t block_threads, DType dtype, int *per_cu);
+// cooperative: hipLaunchCooperativeKernel instead of a plain launch.
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks, uint32_t block_threads, WireArgs &args,
-                       int cooperative, int cus, DType dtype);
+                       uint32_t blocks, uint32_t block_threads, WireArgs &args, bool cooperative,
+                       DType dtype);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
 // The library's own fixed scratch region in device memory (one per GPU, held
 // until the process ends): its device address on the current device and its size.

@@ -11,7 +11,7 @@
 // 57-81,112-206 (Sequential), 262-278,333-516 (Ring), simple_transmit.hpp:16-179
 // and bisect_transmit.hpp:286-424,432-481, re-tiled for 64-lane wavefronts.
 //
-// Four wire formats:
+// Five wire formats:
 //   WireLL    (Rt64, rt64.hpp:334-341): every 8-byte store carries 4 bytes
 //             of payload and the 4-byte flag, so a message validates itself; the
 //             receiver re-polls until a wave-wide vote says every lane's flag is
@@ -19,8 +19,11 @@
 //             Needs nothing but 8-byte store atomicity.
 //   WireLL16  (Rt64_PCIE, rt64.hpp:3-20): 16-byte stores of 8 bytes of payload and
 //             the flag twice.
-//   WireLL64  (Rt64_128 family): 15 payload dwords + 1 flag per 64-byte segment.
-//   WireFlag  (assumption-free alternative for the Rt64_128 family): payload lines
+//   WireRt128 (Rt64_128, rt64_128.hpp:538-553): the reference's 128-byte message,
+//             30 payload dwords and a flag in each 64-byte half, byte for byte.
+//   WireRt256 (Rt64_128_PCIE, rt64_128.hpp:3-30): the reference's 256-byte message,
+//             60 payload dwords and a flag in each 64-byte quarter, byte for byte.
+//   WireFlag  (assumption-free alternative for the Rt64_128 families): payload lines
 //             plus a separate flag word, ordered by agent-scope release/acquire
 //             fences.
 //
@@ -108,6 +111,44 @@ struct Spin {
 
 // ---- wire formats ---------------------------------------------------------------
 
+// Every embedded-flag format ends a slot with a flag word (the last lane's last
+// dword).  A wave first reads the whole messages (one round trip when they are
+// already there).  If some flag is still old it stops re-reading payload and
+// watches just that last word of each message: lane i < M loads the last dword
+// of slot i, so an unsuccessful look costs one 4-byte access per message.  The
+// full read that follows again checks every flag of every message.
+template <int M>
+static __device__ __forceinline__ bool await_last_flags(const char *const (&slot)[M], uint32_t slot_bytes,
+                                                        uint32_t flag, uint32_t lane, Spin &spin) {
+  static_assert(M <= 64, "one lane per message");
+  if (spin.dead) return false;
+  const char *mine = slot[0];
+#pragma unroll
+  for (int i = 1; i < M; ++i) mine = lane == (uint32_t)i ? slot[i] : mine;
+  const uint32_t *word = reinterpret_cast<const uint32_t *>(mine + slot_bytes - 4);
+  uint32_t polls = 0;
+  for (;;) {
+    const bool ok = lane >= (uint32_t)M || __hip_atomic_load(word, __ATOMIC_RELAXED, VR_AGENT) == flag;
+    if (__all(ok)) return true;
+    if (spin.give_up(polls)) return false;
+  }
+}
+
+// Row-wise lane moves inside each group of 16 lanes (a DPP row): lane i receives
+// the value of lane i - N (shift right) or i + N (shift left); lanes without a
+// source keep `old`.
+template <int N>
+static __device__ __forceinline__ uint32_t row_shr(uint32_t old, uint32_t src) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, 0x110 + N, 0xf, 0xf, false);
+}
+template <int N>
+static __device__ __forceinline__ uint32_t row_shl(uint32_t old, uint32_t src) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, 0x100 + N, 0xf, 0xf, false);
+}
+
+constexpr uint32_t kOffNowhere = 0x7ffffff0u;   // beyond any buffer: loads give 0, stores are dropped
+
+
 template <int U, int DT>
 struct WireLL {
   static constexpr uint32_t kWireBytes = 64u * 4u * U;   // payload one wave moves per step
@@ -149,6 +190,7 @@ struct WireLL {
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
                                               uint32_t flag, uint32_t lane, Spin &spin) {
     if (spin.dead) return false;
+    const char *const one[1] = {slot};
     uint32_t polls = 0;
     for (;;) {
       bool ok = true;
@@ -157,10 +199,10 @@ struct WireLL {
         const uint64_t msg = __hip_atomic_load(reinterpret_cast<const uint64_t *>(slot) + u * 64 + lane,
                                                __ATOMIC_RELAXED, VR_AGENT);
         v.d[u] = (uint32_t)msg;
-        ok = ok && (uint32_t)(msg >> 32) == flag;
+        ok = ok & ((uint32_t)(msg >> 32) == flag);
       }
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     }
   }
   // M messages at once: all loads are in flight together, so the wait costs one
@@ -180,10 +222,10 @@ struct WireLL {
           const uint64_t msg = __hip_atomic_load(
               reinterpret_cast<const uint64_t *>(slot[i]) + u * 64 + lane, __ATOMIC_RELAXED, VR_AGENT);
           v[i].d[u] = (uint32_t)msg;
-          ok = ok && (uint32_t)(msg >> 32) == flag;
+          ok = ok & ((uint32_t)(msg >> 32) == flag);
         }
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<M>(slot, kSlotBytes, flag, lane, spin)) return false;
     }
   }
 };
@@ -251,6 +293,7 @@ struct WireLL16 {
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
                                               uint32_t flag, uint32_t lane, Spin &spin) {
     if (spin.dead) return false;
+    const char *const one[1] = {slot};
     const __amdgpu_buffer_rsrc_t rs = rsrc(slot);
     uint32_t polls = 0;
     for (;;) {
@@ -260,10 +303,10 @@ struct WireLL16 {
         const u32x4 msg = __builtin_amdgcn_raw_buffer_load_b128(rs, (u * 64u + lane) * 16u, 0, kAuxAgentVolatile);
         v.d[u][0] = msg.x;
         v.d[u][1] = msg.y;
-        ok = ok && msg.z == flag && msg.w == flag;
+        ok = ok & (msg.z == flag) & (msg.w == flag);
       }
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     }
   }
   template <int M>
@@ -282,95 +325,107 @@ struct WireLL16 {
           const u32x4 msg = __builtin_amdgcn_raw_buffer_load_b128(rs, (u * 64u + lane) * 16u, 0, kAuxAgentVolatile);
           v[i].d[u][0] = msg.x;
           v[i].d[u][1] = msg.y;
-          ok = ok && msg.z == flag && msg.w == flag;
+          ok = ok & (msg.z == flag) & (msg.w == flag);
         }
       }
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<M>(slot, kSlotBytes, flag, lane, spin)) return false;
     }
   }
 };
 
-// Rt64_128 re-tiled for wavefronts (rt64_128.hpp:538-553, 635-685, 724-802): the
-// reference packs 30 payload dwords and a flag at dword 15 and at dword 31 into a
-// 128-byte message, one flag per 64-byte half "because a 128-byte transaction is
-// not atomic across HBM channels".  Here a wave's message is 512 bytes = eight
-// 64-byte segments; the eight lanes of a segment store 8 bytes each in ONE store
-// instruction, lanes 0..6 two payload dwords, lane 7 one payload dword and the
-// flag: 15 payload dwords + 1 flag per 64 bytes, the reference's 93.75 %.  A
-// receiver's lane trusts its segment once the segment's flag lane has seen the
-// expected flag (wave vote).  Like the reference's format this rests on a
-// 64-byte segment written by one instruction becoming visible as a whole.
+// Rt64_128 at sub-group size 16 (rt64_128.hpp:538-553, 635-685, 724-802), byte for
+// byte: a 128-byte message is sixteen 8-byte lanes; lanes 0..14 load 120
+// contiguous payload bytes; shuffleData parks payload dword 15 (lane 7's second
+// dword) in dword 30 (lane 15's first dword); insertFlags writes the flag to
+// dwords 15 and 31, one per 64-byte half "because a 128-byte transaction is not
+// atomic across HBM channels".  A 64-lane wave carries four such messages side by
+// side per instruction (rows of 16 lanes), so a slot is U x 4 reference messages
+// over U x 480 consecutive payload bytes.  A receiver accepts a message once
+// every flag lane has seen the expected flag (wave vote).  Like the reference's
+// format this rests on a 64-byte half written by one store instruction becoming
+// visible as a whole.
 template <int U, int DT>
-struct WireLL64 {
+struct WireRt128 {
   static constexpr uint32_t kWireBytes = 480u * U;
   static constexpr uint32_t kSlotBytes = 512u * U;
   struct Reg {
     uint32_t d[U][2];
   };
-  // Index of the lane's first payload dword inside message u.
-  static __device__ __forceinline__ uint32_t dword0(int u, uint32_t lane) {
-    return (uint32_t)u * 120u + (lane >> 3) * 15u + (lane & 7u) * 2u;
+  // Byte offset of the lane's 8 payload bytes inside the wire (lane 15 of a row: none).
+  static __device__ __forceinline__ uint32_t io_off(int u, uint32_t lane) {
+    return (lane & 15u) == 15u ? kOffNowhere : (uint32_t)u * 480u + (lane >> 4) * 120u + (lane & 15u) * 8u;
   }
   static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
-    const bool two = (lane & 7u) != 7u;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t i = dword0(u, lane);
-      r.d[u][0] = io_ld32(rs, 4u * i, nt);
-      r.d[u][1] = two ? io_ld32(rs, 4u * (i + 1), nt) : 0u;
+      const io_u32x2 z = io_ld64(rs, io_off(u, lane), nt);
+      r.d[u][0] = z.x;
+      r.d[u][1] = z.y;
     }
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
                                                bool nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
-    const bool two = (lane & 7u) != 7u;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t i = dword0(u, lane);
-      io_st32(rs, 4u * i, r.d[u][0], nt);
-      if (two) io_st32(rs, 4u * (i + 1), r.d[u][1], nt);
+      const io_u32x2 z = {r.d[u][0], r.d[u][1]};
+      io_st64(rs, io_off(u, lane), z, nt);
     }
   }
   static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:947-957
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {   // the flag lane's second dword is rewritten by send()
+      for (int k = 0; k < 2; ++k) {   // lane 15 adds leftovers; send() rewrites both of its dwords
         const h2 s = vadd<DT>(__builtin_bit_cast(h2, m.d[u][k]), __builtin_bit_cast(h2, v.d[u][k]));
         v.d[u][k] = __builtin_bit_cast(uint32_t, s);
       }
   }
   static __device__ __forceinline__ void send(char *slot, uint32_t *, const Reg &v, uint32_t flag,
                                               uint32_t lane) {
-    const bool flag_lane = (lane & 7u) == 7u;
+    const uint32_t l = lane & 15u;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint64_t msg = (uint64_t)v.d[u][0] | ((uint64_t)(flag_lane ? flag : v.d[u][1]) << 32);
-      __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, msg, __ATOMIC_RELAXED,
-                         VR_AGENT);
+      const uint32_t parked = row_shr<8>(0u, v.d[u][1]);                 // lane 15 <- lane 7's second dword
+      const uint32_t x = l == 15u ? parked : v.d[u][0];                  // shuffleData
+      const uint32_t y = (l == 7u || l == 15u) ? flag : v.d[u][1];       // insertFlags
+      __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, (uint64_t)x | ((uint64_t)y << 32),
+                         __ATOMIC_RELAXED, VR_AGENT);
     }
+  }
+  // All loads of a poll are issued before any of them is looked at, so that a
+  // poll costs one memory round trip however many messages it covers.
+  static __device__ __forceinline__ uint64_t fetch(const char *slot, int u, uint32_t lane) {
+    return __hip_atomic_load(reinterpret_cast<const uint64_t *>(slot) + u * 64 + lane, __ATOMIC_RELAXED,
+                             VR_AGENT);
+  }
+  // Unpacks message u into v, undoing the shuffle; false if a flag lane saw another flag.
+  static __device__ __forceinline__ bool decode(uint64_t msg, int u, Reg &v, uint32_t flag, uint32_t lane) {
+    const uint32_t l = lane & 15u;
+    const uint32_t x = (uint32_t)msg, y = (uint32_t)(msg >> 32);
+    const uint32_t back = row_shl<8>(0u, x);                             // lane 7 <- lane 15's first dword
+    v.d[u][0] = x;
+    v.d[u][1] = l == 7u ? back : y;                                      // restoreData
+    return ((l & 7u) != 7u) | (y == flag);
   }
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
                                               uint32_t flag, uint32_t lane, Spin &spin) {
     if (spin.dead) return false;
-    const bool flag_lane = (lane & 7u) == 7u;
+    const char *const one[1] = {slot};
     uint32_t polls = 0;
     for (;;) {
+      uint64_t raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) raw[u] = fetch(slot, u, lane);
       bool ok = true;
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint64_t msg = __hip_atomic_load(reinterpret_cast<const uint64_t *>(slot) + u * 64 + lane,
-                                               __ATOMIC_RELAXED, VR_AGENT);
-        v.d[u][0] = (uint32_t)msg;
-        v.d[u][1] = (uint32_t)(msg >> 32);
-        ok = ok && (!flag_lane || v.d[u][1] == flag);
-      }
+      for (int u = 0; u < U; ++u) ok = ok & decode(raw[u], u, v, flag, lane);
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     }
   }
   template <int M>
@@ -378,22 +433,140 @@ struct WireLL64 {
                                                    const uint32_t *const (&)[M], Reg (&v)[M],
                                                    uint32_t flag, uint32_t lane, Spin &spin) {
     if (spin.dead) return false;
-    const bool flag_lane = (lane & 7u) == 7u;
     uint32_t polls = 0;
     for (;;) {
+      uint64_t raw[M][U];
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[i][u] = fetch(slot[i], u, lane);
       bool ok = true;
 #pragma unroll
       for (int i = 0; i < M; ++i)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const uint64_t msg = __hip_atomic_load(
-              reinterpret_cast<const uint64_t *>(slot[i]) + u * 64 + lane, __ATOMIC_RELAXED, VR_AGENT);
-          v[i].d[u][0] = (uint32_t)msg;
-          v[i].d[u][1] = (uint32_t)(msg >> 32);
-          ok = ok && (!flag_lane || v[i].d[u][1] == flag);
-        }
+        for (int u = 0; u < U; ++u) ok = ok & decode(raw[i][u], u, v[i], flag, lane);
       if (__all(ok)) return true;
-      if (spin.give_up(polls)) return false;
+      if (spin.give_up(polls) || !await_last_flags<M>(slot, kSlotBytes, flag, lane, spin)) return false;
+    }
+  }
+};
+
+// Rt64_128_PCIE at sub-group size 16 (rt64_128.hpp:3-30, 101-233), byte for byte:
+// a 256-byte message is sixteen 16-byte lanes; lanes 0..14 load 240 contiguous
+// payload bytes; insertFlags writes the flag to the last dword of lanes 3, 7, 11
+// and 15 (dwords 15, 31, 47, 63: one per 64 bytes); shuffleData parks the payload
+// dwords displaced from 15, 31 and 47 in lane 15's first three dwords (60, 61,
+// 62).  A wave carries four messages per instruction.  Moved with 128-bit buffer
+// instructions at agent scope.
+template <int U, int DT>
+struct WireRt256 {
+  static constexpr uint32_t kWireBytes = 960u * U;
+  static constexpr uint32_t kSlotBytes = 1024u * U;
+  static constexpr int kAuxAgent = 16;                             // sc1
+  static constexpr int kAuxAgentVolatile = (int)0x80000010u;       // sc1, never hoisted or merged
+  struct Reg {
+    uint32_t d[U][4];
+  };
+  static __device__ __forceinline__ uint32_t io_off(int u, uint32_t lane) {
+    return (lane & 15u) == 15u ? kOffNowhere : (uint32_t)u * 960u + (lane >> 4) * 240u + (lane & 15u) * 16u;
+  }
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+    Reg r;
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const io_u32x4 z = io_ld128(rs, io_off(u, lane), nt);
+      r.d[u][0] = z.x;
+      r.d[u][1] = z.y;
+      r.d[u][2] = z.z;
+      r.d[u][3] = z.w;
+    }
+    return r;
+  }
+  static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
+                                               bool nt) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const io_u32x4 z = {r.d[u][0], r.d[u][1], r.d[u][2], r.d[u][3]};
+      io_st128(rs, io_off(u, lane), z, nt);
+    }
+  }
+  static __device__ __forceinline__ void add(Reg &v, const Reg &m) {   // rt64_128.hpp:516-524
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const h2 s = vadd<DT>(__builtin_bit_cast(h2, m.d[u][k]), __builtin_bit_cast(h2, v.d[u][k]));
+        v.d[u][k] = __builtin_bit_cast(uint32_t, s);
+      }
+  }
+  static __device__ __forceinline__ void send(char *slot, uint32_t *, const Reg &v, uint32_t flag,
+                                              uint32_t lane) {
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot, kSlotBytes);
+    const uint32_t l = lane & 15u;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // shuffleData: lane 15 collects the last dwords of lanes 3, 7 and 11
+      const uint32_t p3 = row_shr<12>(0u, v.d[u][3]), p7 = row_shr<8>(0u, v.d[u][3]),
+                     p11 = row_shr<4>(0u, v.d[u][3]);
+      const bool last = l == 15u;
+      const io_u32x4 msg = {last ? p3 : v.d[u][0], last ? p7 : v.d[u][1], last ? p11 : v.d[u][2],
+                            (l & 3u) == 3u ? flag : v.d[u][3]};            // insertFlags
+      __builtin_amdgcn_raw_buffer_store_b128(msg, rs, (u * 64u + lane) * 16u, 0, kAuxAgent);
+    }
+  }
+  static __device__ __forceinline__ io_u32x4 fetch(__amdgpu_buffer_rsrc_t rs, int u, uint32_t lane) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, (u * 64u + lane) * 16u, 0, kAuxAgentVolatile);
+  }
+  static __device__ __forceinline__ bool decode(io_u32x4 msg, int u, Reg &v, uint32_t flag, uint32_t lane) {
+    const uint32_t l = lane & 15u;
+    // restoreData: lanes 3, 7 and 11 take their last dword back from lane 15
+    const uint32_t b3 = row_shl<12>(0u, msg.x), b7 = row_shl<8>(0u, msg.y), b11 = row_shl<4>(0u, msg.z);
+    v.d[u][0] = msg.x;
+    v.d[u][1] = msg.y;
+    v.d[u][2] = msg.z;
+    v.d[u][3] = l == 3u ? b3 : l == 7u ? b7 : l == 11u ? b11 : msg.w;
+    return ((l & 3u) != 3u) | (msg.w == flag);
+  }
+  static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
+                                              uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    const char *const one[1] = {slot};
+    const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot, kSlotBytes);
+    uint32_t polls = 0;
+    for (;;) {
+      io_u32x4 raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) raw[u] = fetch(rs, u, lane);
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < U; ++u) ok = ok & decode(raw[u], u, v, flag, lane);
+      if (__all(ok)) return true;
+      if (spin.give_up(polls) || !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
+    }
+  }
+  template <int M>
+  static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
+                                                   const uint32_t *const (&)[M], Reg (&v)[M],
+                                                   uint32_t flag, uint32_t lane, Spin &spin) {
+    if (spin.dead) return false;
+    uint32_t polls = 0;
+    for (;;) {
+      io_u32x4 raw[M][U];
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot[i], kSlotBytes);
+#pragma unroll
+        for (int u = 0; u < U; ++u) raw[i][u] = fetch(rs, u, lane);
+      }
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int u = 0; u < U; ++u) ok = ok & decode(raw[i][u], u, v[i], flag, lane);
+      if (__all(ok)) return true;
+      if (spin.give_up(polls) || !await_last_flags<M>(slot, kSlotBytes, flag, lane, spin)) return false;
     }
   }
 };
@@ -468,7 +641,7 @@ struct WireFlag {
       bool ok = true;
 #pragma unroll
       for (int i = 0; i < M; ++i)
-        ok = ok && __hip_atomic_load(flagword[i], __ATOMIC_RELAXED, VR_AGENT) == flag;
+        ok = ok & (__hip_atomic_load(flagword[i], __ATOMIC_RELAXED, VR_AGENT) == flag);
       if (ok) break;                       // same words in every lane: wave-uniform
       if (spin.give_up(polls)) return false;
     }
@@ -522,7 +695,7 @@ static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, 
 // N waves per wire column; wave y serves chunk y.  The wave with y == rank owns
 // the column's reduction for its rank's chunk.
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_parallel(WireArgs a) {
   constexpr uint32_t NSLOT = wl::kSlotsFlat;
   const uint32_t kAhead = a.ahead;   // 1 ... NSLOT - 2, checked by the host
   VR_WAVE_PROLOGUE;
@@ -588,7 +761,7 @@ __global__ __launch_bounds__(1024) void k_wire_parallel(WireArgs a) {
 // ---- SequentialTransmit::run (sequential_transmit.hpp:83-207) -----------------------------
 // One wave does everything its rank owes a wire column, peer after peer.
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_sequential(WireArgs a) {
   constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
   const Sinks<W> sk{a};
@@ -645,7 +818,7 @@ __global__ __launch_bounds__(1024) void k_wire_sequential(WireArgs a) {
 // number of wires per rank, so a ring position is only ever reused by the wave
 // that used it before.
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_simple(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_simple(WireArgs a) {
   constexpr uint32_t kPerSection = wl::kSimplePerSection;
   VR_WAVE_PROLOGUE;
   const Sinks<W> sk{a};
@@ -697,7 +870,7 @@ __global__ __launch_bounds__(1024) void k_wire_simple(WireArgs a) {
 
 // ---- RingTransmit::runAllreduce (sequential_transmit.hpp:429-472) ----------------------------
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_ring(WireArgs a) {
   constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
   const Sinks<W> sk{a};
@@ -749,7 +922,7 @@ __global__ __launch_bounds__(1024) void k_wire_ring(WireArgs a) {
 // ---- RingTransmit::runAllgather (sequential_transmit.hpp:474-516) ----------------------------
 // chunk = bytes of one rank's slice; out[r] holds N slices.
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_allgather(WireArgs a) {
   constexpr uint32_t NSLOT = wl::kSlotsRing;
   VR_WAVE_PROLOGUE;
   const Sinks<W> sk{a};
@@ -785,7 +958,7 @@ __global__ __launch_bounds__(1024) void k_wire_allgather(WireArgs a) {
 // ranks the second; pair exchange first, then the flat exchange among the ranks
 // of the same parity.
 template <int N, typename W>
-__global__ __launch_bounds__(1024) void k_wire_bisect(WireArgs a) {
+__global__ __launch_bounds__(256) void k_wire_bisect(WireArgs a) {
   constexpr uint32_t NSLOT = wl::kSlotsFlat;
   constexpr int B = N / 2;
   VR_WAVE_PROLOGUE;
@@ -880,12 +1053,14 @@ __global__ void k_wire_clear(uint64_t *p, size_t n64) {
 // Messages per lane and step for each format; every slot stays within 2 KiB.
 constexpr int kUnrollLL = 4;     // 1 KiB payload in a 2 KiB message
 constexpr int kUnrollLL16 = 2;   // 1 KiB payload in a 2 KiB message
-constexpr int kUnrollLL64 = 4;   // 1920 B payload in a 2 KiB message
+constexpr int kUnrollRt128 = 4;  // 1920 B payload in a 2 KiB slot (sixteen 128-byte messages)
+constexpr int kUnrollRt256 = 2;  // 1920 B payload in a 2 KiB slot (eight 256-byte messages)
 constexpr int kUnrollFlag = 2;   // 2 KiB payload (16-byte lanes), flag word elsewhere
 
 static_assert(WireLL<kUnrollLL, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 static_assert(WireLL16<kUnrollLL16, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
-static_assert(WireLL64<kUnrollLL64, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireRt128<kUnrollRt128, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireRt256<kUnrollRt256, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 static_assert(WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 
 // ---- the library's own scratch -----------------------------------------------------------
@@ -918,10 +1093,9 @@ hipError_t wire_static_scratch(int device, void **ptr, size_t *bytes) {
 
 // ---- host side --------------------------------------------------------------------------
 
+// The kernel of a flow for a wire format W.
 template <typename W>
-static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 grid, dim3 block,
-                              WireArgs &args, int cooperative, int cus) {
-  void *kargs[] = {&args};
+static const void *flow_kernel(WireFlow flow, int nranks) {
   const void *fn = nullptr;
 #define VR_PICK(NN)                                                                         \
   case NN:                                                                                  \
@@ -944,28 +1118,32 @@ static hipError_t launch_flow(hipStream_t s, WireFlow flow, int nranks, dim3 gri
     default: break;
   }
 #undef VR_PICK
-  if (!fn) return hipErrorInvalidValue;
-  // Waves spin on other work-groups' progress, which is only safe when all of
-  // them are resident at once.  The occupancy query says how many work-groups of
-  // this kernel one compute unit holds; a grid within that bound is co-resident
-  // on a device that runs nothing else, and takes the plain launch path (about
-  // 16 us shorter).  A larger grid, or a caller who asks for it, goes through the
-  // cooperative launch, which makes the runtime check the same bound.
-  bool coop = cooperative == 1;
-  if (cooperative < 0) {
-    int per_cu = 0;
-    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, (int)block.x, 0);
-    if (e != hipSuccess) return e;
-    coop = (uint64_t)grid.x > (uint64_t)per_cu * (uint64_t)cus;
+  return fn;
+}
+
+template <int DT>
+static const void *wire_kernel_dt(WireFlow flow, WireFormat fmt, int vec_halves, int nranks) {
+  switch (fmt) {
+    case WIRE_FMT_LL: return flow_kernel<WireLL<kUnrollLL, DT>>(flow, nranks);
+    case WIRE_FMT_RT128: return flow_kernel<WireRt128<kUnrollRt128, DT>>(flow, nranks);
+    case WIRE_FMT_RT256: return flow_kernel<WireRt256<kUnrollRt256, DT>>(flow, nranks);
+    case WIRE_FMT_LL16: return flow_kernel<WireLL16<kUnrollLL16, DT>>(flow, nranks);
+    default:
+      return vec_halves == 8 ? flow_kernel<WireFlag<kUnrollFlag, h8, DT>>(flow, nranks)
+                             : flow_kernel<WireFlag<kUnrollFlag, h4, DT>>(flow, nranks);
   }
-  if (coop) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
-  return hipLaunchKernel(fn, grid, block, kargs, 0, s);
+}
+
+static const void *wire_kernel(WireFlow flow, WireFormat fmt, int vec_halves, int nranks, DType dtype) {
+  return dtype == DT_BF16 ? wire_kernel_dt<DT_BF16>(flow, fmt, vec_halves, nranks)
+                          : wire_kernel_dt<DT_F16>(flow, fmt, vec_halves, nranks);
 }
 
 uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   switch (fmt) {
     case WIRE_FMT_LL: return WireLL<kUnrollLL, DT_F16>::kWireBytes;
-    case WIRE_FMT_LL64: return WireLL64<kUnrollLL64, DT_F16>::kWireBytes;
+    case WIRE_FMT_RT128: return WireRt128<kUnrollRt128, DT_F16>::kWireBytes;
+    case WIRE_FMT_RT256: return WireRt256<kUnrollRt256, DT_F16>::kWireBytes;
     case WIRE_FMT_LL16: return WireLL16<kUnrollLL16, DT_F16>::kWireBytes;
     default:
       return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16>::kWireBytes
@@ -973,28 +1151,28 @@ uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
   }
 }
 
-template <int DT>
-static hipError_t launch_wire_dt(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves,
-                                 int nranks, dim3 grid, dim3 block, WireArgs &args, int cooperative,
-                                 int cus) {
-  if (fmt == WIRE_FMT_LL)
-    return launch_flow<WireLL<kUnrollLL, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
-  if (fmt == WIRE_FMT_LL64)
-    return launch_flow<WireLL64<kUnrollLL64, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
-  if (fmt == WIRE_FMT_LL16)
-    return launch_flow<WireLL16<kUnrollLL16, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
-  if (vec_halves == 8)
-    return launch_flow<WireFlag<kUnrollFlag, h8, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
-  return launch_flow<WireFlag<kUnrollFlag, h4, DT>>(s, flow, nranks, grid, block, args, cooperative, cus);
+// Waves spin on other work-groups' progress, which is only safe when all of them
+// are resident at once.  The occupancy query says how many work-groups of the
+// flow's kernel one compute unit holds; the host keeps every grid within that
+// bound, so it is co-resident on a device that runs nothing else.
+hipError_t wire_blocks_per_cu(WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
+                              uint32_t block_threads, DType dtype, int *per_cu) {
+  const void *fn = wire_kernel(flow, fmt, vec_halves, nranks, dtype);
+  if (!fn) return hipErrorInvalidValue;
+  return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, (int)block_threads, 0);
 }
 
+// cooperative: a cooperative launch makes the runtime check co-residency once
+// more; the plain launch path is about 16 us shorter.
 hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_halves, int nranks,
-                       uint32_t blocks, uint32_t block_threads, WireArgs &args, int cooperative,
-                       int cus, DType dtype) {
+                       uint32_t blocks, uint32_t block_threads, WireArgs &args, bool cooperative,
+                       DType dtype) {
+  const void *fn = wire_kernel(flow, fmt, vec_halves, nranks, dtype);
+  if (!fn) return hipErrorInvalidValue;
+  void *kargs[] = {&args};
   const dim3 grid(blocks), block(block_threads);
-  if (dtype == DT_BF16)
-    return launch_wire_dt<DT_BF16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative, cus);
-  return launch_wire_dt<DT_F16>(s, flow, fmt, vec_halves, nranks, grid, block, args, cooperative, cus);
+  if (cooperative) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+  return hipLaunchKernel(fn, grid, block, kargs, 0, s);
 }
 
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {

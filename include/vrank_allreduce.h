@@ -223,13 +223,15 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch
  * covers; chunks longer than this, at most 1 GiB, take several launches);
- * for the wire transport "wire_fenced" (1 = the Rt64_128 family sends payload
- * lines with a separate flag word ordered by agent-scope release/acquire fences
- * instead of 64-byte segments with an embedded flag) and
- * "wire_cooperative" (0 = plain launch, 1 = cooperative launch; by default a plain
- * launch whenever the occupancy query proves the grid co-resident),
+ * for the wire transport "wire_fenced" (the Rt64_128 families: 1 = payload lines
+ * with a separate flag word ordered by agent-scope release/acquire fences, 2 =
+ * self-validating 8-byte messages, instead of the reference's 128 / 256-byte
+ * messages with a flag in every 64 bytes) and
+ * "wire_cooperative" (1 = cooperative launch; by default a plain launch: the
+ * library sizes every grid within the occupancy query's bound, so it is
+ * co-resident on an otherwise idle device),
  * "wire_stream_io" (1 = inputs loaded and outputs stored with streaming cache
- * policies; default 0 = cached, which measured faster at every size),
+ * policies, 0 = cached; by default streaming from 256 MiB of inputs + outputs on),
  * "wire_ahead" (1..6 steps the parallel flow's scatters run ahead of its gathers),
  * "wire_msg16" (0 = the Rt64_PCIE family sends self-validating 8-byte messages
  * instead of 16-byte stores that carry the flag twice) and

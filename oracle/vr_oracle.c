@@ -465,37 +465,115 @@ static wire_fmt make_fmt(int wire) {
   return f;
 }
 
-/* Pack `cap_dw` payload dwords + flag into a 32-dword message.
- * RT64    : lane l stores {data_l, flag} at dwords 2l, 2l+1 (rt64.hpp:335-337,566-583).
- * RT64_128: dwords 0..14,16..29 payload in place, payload dword 15 parked at 30,
- *           flag at dwords 15 and 31 (rt64_128.hpp:544-553,635-685,724-762). */
+/* Dwords of one message: 128 bytes (Rt64, Rt64_128) or 256 bytes (the *_PCIE formats). */
+static int fmt_msg_dw(int wire) { return fmt_is_pcie(wire) ? 64 : 32; }
+
+/* Pack `cap_dw` payload dwords + flag into one message, byte for byte as the device
+ * code of the reference lays it out at sub-group size 16 (lane l owns dwords
+ * [l * k, l * k + k) of the message, k = dwords per lane):
+ * RT64         : lane l stores {data_l, flag}: dwords 2l, 2l+1 (rt64.hpp:335-337, 566-583).
+ * RT64_PCIE    : lane l stores {d_2l, d_2l+1, flag, flag}: dwords 4l .. 4l+3 (rt64.hpp:3-20,
+ *                61-98: insertFlags writes the last two components of every lane).
+ * RT64_128     : dwords 0..14, 16..29 payload in place, payload dword 15 parked at 30,
+ *                flag at dwords 15 and 31 (rt64_128.hpp:544-553, 635-685, 724-762; the dead
+ *                verifier agrees: temp[30] = temp[15]; temp[15] = flag; temp[31] = flag,
+ *                allreduce.cpp:71, 131-133).
+ * RT64_128_PCIE: 60 payload dwords; flag in the last component of lanes 3, 7, 11, 15 =
+ *                dwords 15, 31, 47, 63; the payload dwords displaced from 15, 31, 47 are
+ *                parked in lane 15's components 0, 1, 2 = dwords 60, 61, 62
+ *                (rt64_128.hpp:7-13, 101-117, 194-203). */
 static void pack_msg(const wire_fmt *f, uint32_t *msg, const uint32_t *payload, uint32_t flag) {
-  if (f->wire == VRO_WIRE_RT64) {
-    for (int l = 0; l < SG; ++l) {
-      msg[2 * l] = payload[l];
-      msg[2 * l + 1] = flag;
-    }
-  } else {
-    for (int k = 0; k < 30; ++k) msg[k] = payload[k];
-    msg[30] = payload[15];
-    msg[15] = flag;
-    msg[31] = flag;
+  switch (f->wire) {
+    case VRO_WIRE_RT64:
+      for (int l = 0; l < SG; ++l) {
+        msg[2 * l] = payload[l];
+        msg[2 * l + 1] = flag;
+      }
+      break;
+    case VRO_WIRE_RT64_PCIE:
+      for (int l = 0; l < SG; ++l) {
+        msg[4 * l] = payload[2 * l];
+        msg[4 * l + 1] = payload[2 * l + 1];
+        msg[4 * l + 2] = flag;
+        msg[4 * l + 3] = flag;
+      }
+      break;
+    case VRO_WIRE_RT64_128:
+      for (int k = 0; k < 30; ++k) msg[k] = payload[k];
+      msg[30] = payload[15];
+      msg[15] = flag;
+      msg[31] = flag;
+      break;
+    default:
+      for (int k = 0; k < 60; ++k) msg[k] = payload[k];
+      msg[60] = payload[15];
+      msg[61] = payload[31];
+      msg[62] = payload[47];
+      msg[15] = msg[31] = msg[47] = msg[63] = flag;
+      break;
   }
 }
 
 /* Returns 0 and the payload when every flag position matches, else -1. */
 static int unpack_msg(const wire_fmt *f, const uint32_t *msg, uint32_t *payload, uint32_t flag) {
-  if (f->wire == VRO_WIRE_RT64) {
-    for (int l = 0; l < SG; ++l) {
-      if (msg[2 * l + 1] != flag) return -1;
-      payload[l] = msg[2 * l];
-    }
-  } else {
-    if (msg[15] != flag || msg[31] != flag) return -1;
-    for (int k = 0; k < 30; ++k) payload[k] = msg[k];
-    payload[15] = msg[30];
+  switch (f->wire) {
+    case VRO_WIRE_RT64:
+      for (int l = 0; l < SG; ++l) {
+        if (msg[2 * l + 1] != flag) return -1;
+        payload[l] = msg[2 * l];
+      }
+      break;
+    case VRO_WIRE_RT64_PCIE:
+      for (int l = 0; l < SG; ++l) {
+        if (msg[4 * l + 2] != flag || msg[4 * l + 3] != flag) return -1;
+        payload[2 * l] = msg[4 * l];
+        payload[2 * l + 1] = msg[4 * l + 1];
+      }
+      break;
+    case VRO_WIRE_RT64_128:
+      if (msg[15] != flag || msg[31] != flag) return -1;
+      for (int k = 0; k < 30; ++k) payload[k] = msg[k];
+      payload[15] = msg[30];
+      break;
+    default:
+      if (msg[15] != flag || msg[31] != flag || msg[47] != flag || msg[63] != flag) return -1;
+      for (int k = 0; k < 60; ++k) payload[k] = msg[k];
+      payload[15] = msg[60];
+      payload[31] = msg[61];
+      payload[47] = msg[62];
+      break;
   }
   return 0;
+}
+
+int vro_wire_payload_dwords(int wire) {
+  return (wire < VRO_WIRE_RT64 || wire > VRO_WIRE_RT64_128_PCIE) ? -1 : make_fmt(wire).cap_dw;
+}
+int vro_wire_message_dwords(int wire) {
+  return (wire < VRO_WIRE_RT64 || wire > VRO_WIRE_RT64_128_PCIE) ? -1 : fmt_msg_dw(wire);
+}
+int vro_pack_message(int wire, uint32_t *msg, const uint32_t *payload, uint32_t flag) {
+  if (wire < VRO_WIRE_RT64 || wire > VRO_WIRE_RT64_128_PCIE) return -2;
+  const wire_fmt f = make_fmt(wire);
+  pack_msg(&f, msg, payload, flag);
+  return 0;
+}
+int vro_unpack_message(int wire, const uint32_t *msg, uint32_t *payload, uint32_t flag) {
+  if (wire < VRO_WIRE_RT64 || wire > VRO_WIRE_RT64_128_PCIE) return -2;
+  const wire_fmt f = make_fmt(wire);
+  return unpack_msg(&f, msg, payload, flag);
+}
+
+/* A sink cell of the ring / sequential emulators: one packed message. */
+typedef struct {
+  uint32_t msg[64];
+} cell;
+static void cell_send(const wire_fmt *f, cell *c, const uint32_t *payload, uint32_t flag) {
+  pack_msg(f, c->msg, payload, flag);
+}
+static int cell_recv(const wire_fmt *f, const cell *c, uint32_t *payload, uint32_t flag) {
+  memset(payload, 0, sizeof(uint32_t) * MAX_DW);
+  return unpack_msg(f, c->msg, payload, flag);
 }
 
 /* Predicated load of one wire: lanes whose first element index is >= n_left stay 0. */
@@ -627,11 +705,7 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire_kind, 
   const size_t cap = (size_t)f.cap_dw * 4;
   const size_t loop = W * cap;
   enum { NSLOT = 4 };
-  /* sinks: [rank][peer][slot][wire] of {32 payload dwords, flag} */
-  typedef struct {
-    uint32_t p[MAX_DW];
-    uint32_t flag;
-  } cell;
+  /* sinks: [rank][peer][slot][wire] of packed messages */
   const size_t cells = (size_t)N * NSLOT * W;
   cell *scat[MAXR], *gath[MAXR];
   for (int r = 0; r < N; ++r) {
@@ -652,47 +726,39 @@ int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire_kind, 
       /* step 0: rank r sends chunk r to r+1 */
       for (int r = 0; r < N; ++r) {
         const int peer = r, next = (r + 1) % N;
-        cell *c = CELL(scat[next], peer, slot, w);
-        load_wire(&f, c->p, io[r] + (size_t)peer * work_elems + off_el, left);
-        c->flag = flag;
+        load_wire(&f, v, io[r] + (size_t)peer * work_elems + off_el, left);
+        cell_send(&f, CELL(scat[next], peer, slot, w), v, flag);
       }
       /* steps 1..N-2: load chunk (r-i), add what (r-1) sent, forward */
       for (int i = 1; i < N - 1 && rc == 0; ++i)
         for (int r = 0; r < N; ++r) {
           const int peer = (r + N - i) % N, next = (r + 1) % N;
           cell *src = CELL(scat[r], peer, slot, w);
-          if (src->flag != flag) { rc = -1; break; }
+          uint32_t m[MAX_DW];
+          if (cell_recv(&f, src, m, flag)) { rc = -1; break; }
           load_wire(&f, v, io[r] + (size_t)peer * work_elems + off_el, left);
-          accum(v, src->p, f.cap_dw);
-          src->flag = flag - 1;                               /* consumed */
-          cell *dst = CELL(scat[next], peer, slot, w);
-          memcpy(dst->p, v, sizeof v);
-          dst->flag = flag;
+          accum(v, m, f.cap_dw);
+          memset(src, 0, sizeof *src);                        /* consumed */
+          cell_send(&f, CELL(scat[next], peer, slot, w), v, flag);
         }
       /* step N-1: final add for chunk (r+1), push into the gather ring, store */
       for (int r = 0; r < N && rc == 0; ++r) {
         const int peer = (r + 1) % N, next = (r + 1) % N;
-        cell *src = CELL(scat[r], peer, slot, w);
-        if (src->flag != flag) { rc = -1; break; }
+        uint32_t m[MAX_DW];
+        if (cell_recv(&f, CELL(scat[r], peer, slot, w), m, flag)) { rc = -1; break; }
         load_wire(&f, v, io[r] + (size_t)peer * work_elems + off_el, left);
-        accum(v, src->p, f.cap_dw);
-        cell *dst = CELL(gath[next], peer, slot, w);
-        memcpy(dst->p, v, sizeof v);
-        dst->flag = flag;
+        accum(v, m, f.cap_dw);
+        cell_send(&f, CELL(gath[next], peer, slot, w), v, flag);
         store_wire(&f, io[r] + (size_t)peer * work_elems + off_el, v, left);
       }
       /* N-2 forward+store hops, then a last store */
       for (int i = 1; i < N && rc == 0; ++i)
         for (int r = 0; r < N; ++r) {
           const int peer = (r + 1 + N - i) % N, next = (r + 1) % N;   /* p_idx = -(N-1)-i */
-          cell *src = CELL(gath[r], peer, slot, w);
-          if (src->flag != flag) { rc = -1; break; }
-          if (i < N - 1) {
-            cell *dst = CELL(gath[next], peer, slot, w);
-            memcpy(dst->p, src->p, sizeof src->p);
-            dst->flag = flag;
-          }
-          store_wire(&f, io[r] + (size_t)peer * work_elems + off_el, src->p, left);
+          uint32_t m[MAX_DW];
+          if (cell_recv(&f, CELL(gath[r], peer, slot, w), m, flag)) { rc = -1; break; }
+          if (i < N - 1) cell_send(&f, CELL(gath[next], peer, slot, w), m, flag);
+          store_wire(&f, io[r] + (size_t)peer * work_elems + off_el, m, left);
         }
     }
   }
@@ -719,10 +785,6 @@ int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire_
   const size_t cap = (size_t)f.cap_dw * 4;
   const size_t loop = W * cap;
   enum { NSLOT = 4 };
-  typedef struct {
-    uint32_t p[MAX_DW];
-    uint32_t flag;
-  } cell;
   const size_t cells = (size_t)N * NSLOT * W;
   cell *scat[MAXR], *gath[MAXR];
   for (int r = 0; r < N; ++r) {
@@ -743,9 +805,9 @@ int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire_
       for (int r = 0; r < N; ++r)
         for (int i = 0; i < N - 1; ++i) {
           const int next = (r + i + 1) % N;
-          cell *c = CELL(scat[next], r, slot, w);
-          load_wire(&f, c->p, io[r] + (size_t)next * work_elems + off_el, left);
-          c->flag = flag;
+          uint32_t p[MAX_DW];
+          load_wire(&f, p, io[r] + (size_t)next * work_elems + off_el, left);
+          cell_send(&f, CELL(scat[next], r, slot, w), p, flag);
         }
       /* reduce own chunk with the peers' messages in order rank+1, rank+2, ... (l.130-171),
        * gather-push (l.173-177), store (l.181-186) */
@@ -754,16 +816,14 @@ int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire_
         load_wire(&f, v, io[r] + (size_t)r * work_elems + off_el, left);
         for (int i = 0; i < N - 1; ++i) {
           const int next = (r + i + 1) % N;
-          const cell *c = CELL(scat[r], next, slot, w);
-          if (c->flag != flag) { rc = -1; break; }
-          accum(v, c->p, f.cap_dw);
+          uint32_t m[MAX_DW];
+          if (cell_recv(&f, CELL(scat[r], next, slot, w), m, flag)) { rc = -1; break; }
+          accum(v, m, f.cap_dw);
         }
         if (rc) break;
         for (int i = 0; i < N - 1; ++i) {
           const int next = (r + i + 1) % N;
-          cell *c = CELL(gath[next], r, slot, w);
-          memcpy(c->p, v, sizeof v);
-          c->flag = flag;
+          cell_send(&f, CELL(gath[next], r, slot, w), v, flag);
         }
         store_wire(&f, io[r] + (size_t)r * work_elems + off_el, v, left);
       }
@@ -771,9 +831,9 @@ int vro_emulate_sequential(uint16_t *const io[], int nranks, size_t n, int wire_
       for (int r = 0; r < N && rc == 0; ++r)
         for (int i = 0; i < N - 1; ++i) {
           const int next = (r + i + 1) % N;
-          const cell *c = CELL(gath[r], next, slot, w);
-          if (c->flag != flag) { rc = -1; break; }
-          store_wire(&f, io[r] + (size_t)next * work_elems + off_el, c->p, left);
+          uint32_t m[MAX_DW];
+          if (cell_recv(&f, CELL(gath[r], next, slot, w), m, flag)) { rc = -1; break; }
+          store_wire(&f, io[r] + (size_t)next * work_elems + off_el, m, left);
         }
     }
   }
@@ -799,10 +859,6 @@ int vro_emulate_allgather_ring(uint16_t *const out[], const uint16_t *const in[]
   const size_t cap = (size_t)f.cap_dw * 4;
   const size_t loop = W * cap;
   enum { NSLOT = 4 };
-  typedef struct {
-    uint32_t p[MAX_DW];
-    uint32_t flag;
-  } cell;
   const size_t cells = (size_t)N * NSLOT * W;
   cell *gath[MAXR];
   for (int r = 0; r < N; ++r) gath[r] = calloc(cells, sizeof(cell));
@@ -818,24 +874,20 @@ int vro_emulate_allgather_ring(uint16_t *const out[], const uint16_t *const in[]
       /* own slice: store unless the input already is the output slot, send on */
       for (int r = 0; r < N; ++r) {
         const int peer = r, next = (r + 1) % N;
-        cell *c = CELL(gath[next], peer, slot, w);
-        load_wire(&f, c->p, in[r] + off_el, left);
-        c->flag = flag;
+        uint32_t p[MAX_DW];
+        load_wire(&f, p, in[r] + off_el, left);
+        cell_send(&f, CELL(gath[next], peer, slot, w), p, flag);
         uint16_t *o = out[r] + (size_t)peer * work_elems + off_el;
-        if (o != in[r] + off_el) store_wire(&f, o, c->p, left);
+        if (o != in[r] + off_el) store_wire(&f, o, p, left);
       }
       /* p_idx = -1, -2, ...: receive slice (rank - i), forward it except on the last hop */
       for (int i = 1; i < N && rc == 0; ++i)
         for (int r = 0; r < N; ++r) {
           const int peer = (r + N - i) % N, next = (r + 1) % N;
-          const cell *c = CELL(gath[r], peer, slot, w);
-          if (c->flag != flag) { rc = -1; break; }
-          if (i < N - 1) {
-            cell *d = CELL(gath[next], peer, slot, w);
-            memcpy(d->p, c->p, sizeof c->p);
-            d->flag = flag;
-          }
-          store_wire(&f, out[r] + (size_t)peer * work_elems + off_el, c->p, left);
+          uint32_t m[MAX_DW];
+          if (cell_recv(&f, CELL(gath[r], peer, slot, w), m, flag)) { rc = -1; break; }
+          if (i < N - 1) cell_send(&f, CELL(gath[next], peer, slot, w), m, flag);
+          store_wire(&f, out[r] + (size_t)peer * work_elems + off_el, m, left);
         }
     }
   }

@@ -114,13 +114,24 @@ enum {
   VRO_WIRE_RT64_128_PCIE = 3,  /* rt64_128.hpp:3-21  240 B payload / 256 B message (ring, sequential, all-gather) */
 };
 
+/* One message of a wire format, byte for byte as the reference's device code lays it
+ * out at sub-group size 16: `payload` holds vro_wire_payload_dwords(wire) dwords,
+ * `msg` vro_wire_message_dwords(wire) dwords (32 or 64).  Unpack returns -1 when a
+ * flag position does not carry `flag`.  Pinned by hand-derived positions
+ * (rt64.hpp:3-20, 335-341; rt64_128.hpp:7-13, 101-117, 194-203, 544-553, 635-685,
+ * 724-762) and the reference's dead stage verifier (allreduce.cpp:71, 131-133). */
+int vro_wire_payload_dwords(int wire);
+int vro_wire_message_dwords(int wire);
+int vro_pack_message(int wire, uint32_t *msg, const uint32_t *payload, uint32_t flag);
+int vro_unpack_message(int wire, const uint32_t *msg, uint32_t *payload, uint32_t flag);
+
 /* AllReduce<T,N,Proto,ParallelTransmit,16>::operator() for every rank
  * (allreduce.hpp:83-104 + parallel_transmit.hpp:63-131). */
 int vro_emulate_parallel(uint16_t *const io[], int nranks, size_t n, int wire,
                          int groups, int subgroups, uint32_t seq_no);
 
 /* AllReduce<T,N,Proto,RingTransmit,16> (sequential_transmit.hpp:429-472); the
- * wire format does not change the arithmetic so only payload moves here. */
+ * messages travel packed in the wire format's byte layout. */
 int vro_emulate_ring(uint16_t *const io[], int nranks, size_t n, int wire,
                      int groups, int subgroups, uint32_t seq_no);
 

@@ -98,6 +98,15 @@ class Oracle:
         L.vro_emulate_bisect_dt.restype = C.c_int
         L.vro_emulate_bisect_dt.argtypes = [C.c_int, C.POINTER(_u16p), C.c_int, C.c_size_t, C.c_int,
                                             C.c_int, C.c_uint32]
+        _u32p = C.POINTER(C.c_uint32)
+        L.vro_wire_payload_dwords.restype = C.c_int
+        L.vro_wire_payload_dwords.argtypes = [C.c_int]
+        L.vro_wire_message_dwords.restype = C.c_int
+        L.vro_wire_message_dwords.argtypes = [C.c_int]
+        L.vro_pack_message.restype = C.c_int
+        L.vro_pack_message.argtypes = [C.c_int, _u32p, _u32p, C.c_uint32]
+        L.vro_unpack_message.restype = C.c_int
+        L.vro_unpack_message.argtypes = [C.c_int, _u32p, _u32p, C.c_uint32]
         L.vro_set_threads.restype = C.c_int
         L.vro_set_threads.argtypes = [C.c_int]
 
@@ -235,6 +244,29 @@ class Oracle:
         rc = self.lib.vro_emulate_bisect(_ptr_array(io), len(io), len(io[0]), groups, subgroups,
                                          seq_no)
         return rc, io
+
+    def wire_dwords(self, wire):
+        """(payload dwords, message dwords) of one message of the wire format."""
+        return self.lib.vro_wire_payload_dwords(wire), self.lib.vro_wire_message_dwords(wire)
+
+    def pack_message(self, wire, payload, flag):
+        cap, size = self.wire_dwords(wire)
+        payload = np.ascontiguousarray(payload, np.uint32)
+        assert len(payload) == cap
+        msg = np.zeros(size, np.uint32)
+        u32p = C.POINTER(C.c_uint32)
+        rc = self.lib.vro_pack_message(wire, msg.ctypes.data_as(u32p), payload.ctypes.data_as(u32p), flag)
+        assert rc == 0
+        return msg
+
+    def unpack_message(self, wire, msg, flag):
+        cap, size = self.wire_dwords(wire)
+        msg = np.ascontiguousarray(msg, np.uint32)
+        assert len(msg) == size
+        payload = np.zeros(cap, np.uint32)
+        u32p = C.POINTER(C.c_uint32)
+        rc = self.lib.vro_unpack_message(wire, msg.ctypes.data_as(u32p), payload.ctypes.data_as(u32p), flag)
+        return rc, payload
 
     def set_threads(self, n):
         return self.lib.vro_set_threads(n)

@@ -188,6 +188,21 @@ def test_parallel_defaults_to_wire_and_sweep_sizes(ctxs, oracle):
         H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins), "n=%d" % n)
 
 
+@pytest.mark.parametrize("log2_elems", [24, 25, 26, 27])
+def test_config5_parallel_large_sizes(ctxs, oracle, log2_elems):
+    """The sweep's named protocol on its default (wire) transport at 32, 64, 128 and
+    256 MiB per rank: N(0,1) inputs, rank 0 compared in full with the rotated-order
+    oracle, the other ranks by equality with rank 0."""
+    n = 1 << log2_elems
+    ins = H.make_inputs(oracle, 8, n, 5000 + log2_elems)
+    want = oracle.rotated(ins)
+    got, _ = H.run_allreduce(ctxs[8], "parallel", ins)          # default transport = wire
+    assert oracle.count_mismatch(got[0], want) == 0, n
+    for r in range(1, 8):
+        assert oracle.count_mismatch(got[r], got[0]) == 0, (n, r)
+    assert oracle.count_mismatch(want, oracle.rank_order(ins)) > 1000   # the order matters on this data
+
+
 def run_allgather_wire(ctx, algo, ins, alias_own_slot=False):
     from gpu_ipc_example_amd.binding import DeviceBuffer
     N, n = ctx.nranks, len(ins[0])
