@@ -120,6 +120,42 @@ def time_kernels(binding, ctx, name, sets, iters, group=1):
     return out
 
 
+def memory_clock():
+    """The memory clock levels the driver reports (sysfs, `*` marks the current
+    one), sampled while the GPU is still warm from the timed region."""
+    import glob
+    found = {}
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_mclk")):
+        try:
+            lines = [l.strip() for l in open(path).read().splitlines() if l.strip()]
+        except OSError:
+            continue
+        found[path.split("/")[4]] = {"levels": [l.rstrip(" *") for l in lines],
+                                     "current": [l.rstrip(" *") for l in lines if l.endswith("*")]}
+    return found or None
+
+
+def multi_stream_copy(binding, ctx, name, sets, iters, group):
+    """The all-reduce kernel itself with the adds removed (N read streams, N write
+    streams, same grid, addressing and cache policies), on the same rotating
+    buffer sets: the ceiling of this access shape."""
+    n, algo, ne, *_ = WORKLOADS[name]
+    npairs = (iters + group - 1) // group
+    timer = binding.EventTimer(npairs)
+    k = 0
+    for p in range(npairs):
+        timer.start(p)
+        for _ in range(group):
+            ins, outs = sets[k % len(sets)]
+            ctx.stream_probe_multi([b.ptr for b in outs], [b.ptr for b in ins], ne * 2)
+            k += 1
+        timer.stop(p)
+    ctx.sync()
+    ms = timer.elapsed_ms(npairs) / group
+    timer.close()
+    return float(ms.mean())
+
+
 def hbm_ceilings(binding, ctx):
     """Plain streaming kernels over 2 GiB (nothing cache-resident): what this
     GPU's HBM delivers for pure reads, pure writes and a 1:1 copy."""
@@ -370,6 +406,7 @@ def main():
                                len(sets), len(sets) * (B if not args.inplace else B / 2) / 2**20)
                            if len(sets) > 1 else "every step reuses one buffer set (cache-warm)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "memory_clock": memory_clock(),
         "bit_exact_vs_oracle": None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
@@ -418,6 +455,16 @@ def main():
                     "overhead (a kernel trace shows p50 4.2-4.5 us); back_to_back_us: 20 launches per "
                     "event pair, per launch; buffers are cache-resident"}
         result["hbm_ceilings"] = hbm_ceilings(binding, ctx)
+        if sets[0][1] is not None and not algo.startswith("allgather"):
+            # the same kernel, grid and policies without the adds, on the same buffer sets
+            time_kernels(binding, ctx, name, sets, 8)                      # back to steady state
+            c_ms = multi_stream_copy(binding, ctx, name, sets, args.steps, args.event_group)
+            a_ms = float(time_kernels(binding, ctx, name, sets, args.steps, group=args.event_group).mean())
+            result["hbm_ceilings"]["same_shape_no_adds"] = {
+                "kernel_us_avg": round(c_ms * 1e3, 3), "GBps": round(B / (c_ms * 1e-3) / 1e9, 1),
+                "allreduce_us_avg_same_run": round(a_ms * 1e3, 3),
+                "note": "k_direct_allreduce with the adds removed: %d read + %d write streams, same "
+                        "grid, buffer addressing and nt / nt sc1 policies, same rotating buffer sets" % (n, n)}
 
     if want_check:
         result["cpu_baseline"], bad = cpu_leg(name, gpu_results, args.cpu_seconds)

@@ -94,6 +94,10 @@ def lib():
         "vr_time_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_copy": (i, [vp, vp, vp, vp, sz, i, C.POINTER(C.c_float)]),
         "vr_stream_probe": (i, [vp, vp, i, vp, vp, sz]),
+        "vr_stream_probe_multi": (i, [vp, vp, vpp, vpp, sz]),
+        "vr_ipc_open_all": (i, [vp, i, i, vpp, C.POINTER(sz), C.c_char_p]),
+        "vr_ipc_close_all": (i, [i, i, vpp]),
+        "vr_ipc_barrier": (i, [i, i, C.c_char_p, i]),
         "vr_probe_xcc_ids": (i, [vp, u32, C.POINTER(u32)]),
         "vr_fill_pattern": (None, [C.POINTER(C.c_uint16), i, sz]),
         "vr_generate": (None, [C.POINTER(C.c_uint16), sz, C.c_uint64, i, C.c_double, C.c_double]),
@@ -334,6 +338,10 @@ class VirtualRanks:
         """mode: 0 copy, 1 read only, 2 write only."""
         _check(lib().vr_stream_probe(self._h, stream, mode, C.c_void_p(int(dst)),
                                      C.c_void_p(int(src)), nbytes))
+
+    def stream_probe_multi(self, dsts, srcs, nbytes_each, stream=None):
+        """The all-reduce kernel with the adds removed: dsts[k] = srcs[k] for nranks streams."""
+        _check(lib().vr_stream_probe_multi(self._h, stream, _table(dsts), _table(srcs), nbytes_each))
 
     def xcc_ids(self, blocks):
         out = (C.c_uint32 * blocks)()

@@ -24,6 +24,11 @@ static int fail(int status, const std::string &detail) {
   return status;
 }
 
+namespace vr {
+// For the library's other translation units.
+int api_fail(int status, const std::string &detail) { return fail(status, detail); }
+}  // namespace vr
+
 static int fail_hip(hipError_t e, const char *what) {
   return fail(VR_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
 }
@@ -1132,6 +1137,29 @@ extern "C" int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, c
   if (int rc = copy_tuning(ctx, dst, src, bytes, mode, &t)) return rc;
   hipError_t e = launch_copy((hipStream_t)stream, ctx->dev, t, dst, src, bytes, mode);
   return e == hipSuccess ? VR_OK : fail_hip(e, "launch_copy");
+}
+
+extern "C" int vr_stream_probe_multi(vr_ctx *ctx, void *stream, void *const dsts[],
+                                     const void *const srcs[], size_t bytes_each) {
+  if (int rc = use_device(ctx)) return rc;
+  if (!dsts || !srcs) return fail(VR_ERR_INVALID, "null table");
+  const int N = ctx->nranks;
+  if (bytes_each % (16 * (size_t)N)) return fail(VR_ERR_UNEVEN, "bytes per stream must be a multiple of 16 * nranks");
+  PtrTable in, out;
+  memset(&in, 0, sizeof in);
+  memset(&out, 0, sizeof out);
+  for (int r = 0; r < N; ++r) {
+    if (!dsts[r] || !srcs[r]) return fail(VR_ERR_INVALID, "null stream pointer");
+    if ((uintptr_t)dsts[r] % 16 || (uintptr_t)srcs[r] % 16) return fail(VR_ERR_UNALIGNED, "16-byte alignment");
+    in.p[r] = const_cast<void *>(srcs[r]);
+    out.p[r] = dsts[r];
+  }
+  // Exactly the launch an out-of-place all-reduce of this size would get.
+  const size_t all = (size_t)N * bytes_each;
+  const Tuning t = tuning_for(ctx, &kAlgos[VR_ALGO_BISECT], all, all, false);
+  hipError_t e = launch_direct_allreduce((hipStream_t)stream, ctx->dev, t, N, ORDER_COPY, DT_F16, in, out,
+                                         bytes_each / 2 / (size_t)N, 8);
+  return e == hipSuccess ? VR_OK : fail_hip(e, "launch_direct_allreduce (copy yardstick)");
 }
 
 extern "C" int vr_probe_xcc_ids(vr_ctx *ctx, uint32_t blocks, uint32_t *ids_host) {

@@ -64,15 +64,17 @@ __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, uint32_t off, V v) 
 // `owner`, and the chunk index itself.
 template <int N, int ORDER>
 __device__ __forceinline__ int chunk_of_owner(int owner) {
-  if constexpr (ORDER == ORDER_ROTATED)
-    return owner;
-  else
+  if constexpr (ORDER == ORDER_BISECT)
     return (owner & 1) * (N / 2) + (owner >> 1);
+  else
+    return owner;
 }
 
 template <int N, int ORDER>
 __device__ __forceinline__ int operand_rank(int owner, int k) {
-  if constexpr (ORDER == ORDER_ROTATED) {
+  if constexpr (ORDER == ORDER_COPY) {
+    return k;
+  } else if constexpr (ORDER == ORDER_ROTATED) {
     return (owner + k) % N;                       // own chunk first, then rank+1, rank+2, ...
   } else {
     constexpr int B = N / 2;
@@ -132,9 +134,15 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
       for (int k = 0; k < N; ++k) x[u][k] = ld<V, LD_AUX>(src[k], t + u * row + lane);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const V acc = reduce_operands<N, ORDER, DT, V>(x[u]);
+      if constexpr (ORDER == ORDER_COPY) {
+        // the all-reduce's N read streams and N write streams with the adds removed
 #pragma unroll
-      for (int k = 0; k < N; ++k) st<V, ST_AUX>(dst[k], t + u * row + lane, acc);
+        for (int k = 0; k < N; ++k) st<V, ST_AUX>(dst[k], t + u * row + lane, x[u][k]);
+      } else {
+        const V acc = reduce_operands<N, ORDER, DT, V>(x[u]);
+#pragma unroll
+        for (int k = 0; k < N; ++k) st<V, ST_AUX>(dst[k], t + u * row + lane, acc);
+      }
     }
   }
 }
@@ -317,6 +325,10 @@ hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const T
   if (t.block < 64 || t.block > 1024 || t.block % 64) return hipErrorInvalidValue;
 #define VR_CASE(NN)                                                                              \
   case NN:                                                                                       \
+    if (order == ORDER_COPY) {                                                                   \
+      if (vec_halves != 8) return hipErrorInvalidValue;                                          \
+      return launch_ar_unroll<NN, ORDER_COPY, DT_F16, h8>(s, dev, t, in, out, chunk_elems * 2);  \
+    }                                                                                            \
     if (order == ORDER_BISECT) {                                                                 \
       if constexpr (NN >= 4)                                                                     \
         return launch_ar_vec<NN, ORDER_BISECT>(s, dev, t, dtype, in, out, chunk_elems, vec_halves);     \

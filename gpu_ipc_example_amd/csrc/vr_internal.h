@@ -29,6 +29,7 @@ enum DType : int {
 enum Order : int {
   ORDER_ROTATED = 0,  // chain from the chunk owner: parallel/sequential/ring/simple transmit
   ORDER_BISECT = 1,   // pair sums, then chain over pairs: BisectPTransmit
+  ORDER_COPY = 2,     // yardstick: no adds, output k receives input k (same launch shape and traffic)
 };
 
 struct Tuning {

@@ -10,6 +10,13 @@
 //   -t/--transport     direct | wire
 //   -d/--device        HIP device index
 //   --dtype            f16 | bf16 (the reference is built for one test_type, main.cpp:45)
+// and, for the reference's own shape of one process per rank (mpirun -np N ./main):
+//   --rank R           this process is rank R of the -r N ranks; it owns its input and
+//                      scratch, maps every peer's scratch through the IPC exchange
+//                      (main.cpp:241-283, ipc_exchange.cpp) and launches its own wires only
+//   -i/--instance S    socket-name suffix shared by the processes of one run (main.cpp:194)
+//   --seed S           seeded N(0,1) inputs (rank r uses S + r) instead of fill_pattern
+//   --dump FILE        write this rank's result (raw 16-bit elements) to FILE
 // Run protocol (main.cpp:48-109): run #1 with `flag`; with -v verify and return;
 // otherwise two more warm-ups (flag+100, flag+150), then the timed run (flag+200)
 // whose kernel time is printed as "[rank] Running time: <ns>ns" for every rank.
@@ -33,6 +40,10 @@ struct Options {
   uint32_t simd = 16;
   bool verify = false, grid_given = false;
   int ranks = 8, device = 0;
+  int rank = -1;                     // >= 0: one process per rank
+  std::string instance = "0", dump;
+  long long seed = -1;
+  unsigned long long spin = 0;
 };
 
 bool take(int &i, int argc, char **argv, const char *s, const char *l, std::string *out) {
@@ -58,7 +69,8 @@ Options parse(int argc, char **argv) {
       printf("usage: vr_main [-n 8MB] [-r 8] [-a small|simple|bisect|parallel|small_ring|simple_ring|"
              "small_pcie|simple_pcie|small_pcie_p|simple_pcie_p|simple_transmit|allgather_small|allgather_simple]\n"
              "               [-g groups -w subgroups -s simd] [-f flag] [-t direct|wire] [-d device]\n"
-             "               [--dtype f16|bf16] [-v]\n");
+             "               [--dtype f16|bf16] [-v]\n"
+             "               [--rank R -i instance [--seed S] [--dump FILE]]   one process per rank\n");
       exit(0);
     }
     if (take(i, argc, argv, "n", "nelems", &v)) o.nelems = v;
@@ -71,6 +83,11 @@ Options parse(int argc, char **argv) {
     else if (take(i, argc, argv, "t", "transport", &v)) o.transport = v;
     else if (take(i, argc, argv, "d", "device", &v)) o.device = atoi(v.c_str());
     else if (take(i, argc, argv, "D", "dtype", &v)) o.dtype = v;
+    else if (take(i, argc, argv, "R", "rank", &v)) o.rank = atoi(v.c_str());
+    else if (take(i, argc, argv, "i", "instance", &v)) o.instance = v;
+    else if (take(i, argc, argv, "S", "seed", &v)) o.seed = atoll(v.c_str());
+    else if (take(i, argc, argv, "O", "dump", &v)) o.dump = v;
+    else if (take(i, argc, argv, "P", "spin", &v)) o.spin = strtoull(v.c_str(), nullptr, 0);
     // the reference ignores what it does not know (allow_unrecognised_options)
   }
   return o;
@@ -132,6 +149,101 @@ int verify_allgather(const std::vector<std::vector<uint16_t>> &got, int world, s
   return 0;
 }
 
+// One process per rank, the reference's own arrangement (main.cpp:212-314): this
+// process owns rank `o.rank`'s input and its scratch (scatter sink | gather sink,
+// the ipcbuf0 | ipcbuf1 of main.cpp:241-243), zeroes the scratch once, maps every
+// peer's scratch (open_all_ipc_mems, main.cpp:256), builds peerbuf0 / peerbuf1
+// (main.cpp:260-269), waits for all ranks (MPI_Barrier, main.cpp:287) and runs its
+// own wires against them.
+int run_as_rank(const Options &o, int algo, size_t nelems) {
+  const int world = o.ranks, rank = o.rank;
+  if (rank >= world) throw std::invalid_argument("--rank must be below -r");
+  vrank::VirtualRanks ranks(world, o.device);
+  ranks.setDtype(g_dtype);
+  if (o.spin) vrank::check(vr_ctx_set_spin_limit(ranks.get(), o.spin));
+  size_t sink = 0;
+  vrank::check(vr_rank_scratch_bytes(ranks.get(), &sink));
+  const size_t alloc = nelems * sizeof(uint16_t);
+  void *input = nullptr, *scratch = nullptr;
+  vrank::check(vr_malloc(o.device, alloc, &input));
+  vrank::check(vr_malloc(o.device, 2 * sink, &scratch));
+  vrank::check(vr_memset(scratch, 0, 2 * sink));                          // main.cpp:251
+  std::vector<uint16_t> host(nelems);
+  if (o.seed >= 0) vr_generate_dt(g_dtype, host.data(), nelems, (uint64_t)o.seed + (uint64_t)rank, 1, 0.0, 1.0);
+  else vr_fill_pattern_dt(g_dtype, host.data(), rank, nelems);
+  vrank::check(vr_copy_to_device(input, host.data(), alloc));
+
+  void *bases[VR_MAX_RANKS] = {};
+  size_t offsets[VR_MAX_RANKS] = {};
+  vrank::check(vr_ipc_open_all(scratch, rank, world, bases, offsets, o.instance.c_str()));
+  void *peerbuf0[VR_MAX_RANKS] = {}, *peerbuf1[VR_MAX_RANKS] = {};
+  for (int i = 0; i < world; ++i) {
+    peerbuf0[i] = static_cast<char *>(bases[i]) + offsets[i];
+    peerbuf1[i] = static_cast<char *>(peerbuf0[i]) + sink;
+  }
+  int generation = 0;
+  vrank::check(vr_ipc_barrier(rank, world, o.instance.c_str(), ++generation));   // every scratch is zeroed
+
+  void *stream = nullptr;
+  vrank::check(vr_stream_create(o.device, &stream));
+  void *ev0 = nullptr, *ev1 = nullptr;
+  vrank::check(vr_event_create(&ev0));
+  vrank::check(vr_event_create(&ev1));
+  auto run = [&](uint32_t flag) {
+    uint32_t step = flag;
+    vrank::check(vr_allreduce_rank(ranks.get(), stream, algo, rank, input, nullptr, peerbuf0[rank],
+                                   peerbuf1[rank], peerbuf0, peerbuf1, sink, nelems, &step));
+  };
+  int status = 0;
+  run((uint32_t)o.flag);
+  ranks.wait(stream);
+  if (o.verify || !o.dump.empty()) {
+    std::vector<uint16_t> got(nelems);
+    vrank::check(vr_copy_to_host(got.data(), input, alloc));
+    if (!o.dump.empty()) {
+      FILE *f = fopen(o.dump.c_str(), "wb");
+      if (!f || fwrite(got.data(), 2, nelems, f) != nelems) throw std::runtime_error("cannot write " + o.dump);
+      fclose(f);
+    }
+    if (o.verify && o.seed < 0) {
+      // verifyAllReduce for this rank's copy (allreduce.cpp:519-551)
+      std::vector<uint16_t> pattern(nelems), sum(nelems, 0);
+      for (int r = 0; r < world; ++r) {
+        vr_fill_pattern_dt(g_dtype, pattern.data(), r, nelems);
+        for (size_t i = 0; i < nelems; ++i) sum[i] = elem_add(sum[i], pattern[i]);
+      }
+      size_t bad = 0;
+      for (size_t i = 0; i < nelems; ++i)
+        if (sum[i] != got[i] && bad++ < 16)
+          printf("Error Compare! Expected: %g, got: %g@[%d](%zu);\n", elem_value(sum[i]), elem_value(got[i]),
+                 rank, i);
+      if (bad == 0) printf("[%d] verify: %zu elements match the host sum\n", rank, nelems);
+      else printf("[%d] verify: %zu mismatches\n", rank, bad);
+    }
+  } else {
+    run((uint32_t)o.flag + 100);
+    run((uint32_t)o.flag + 150);
+    ranks.wait(stream);
+    vrank::check(vr_ipc_barrier(rank, world, o.instance.c_str(), ++generation));  // main.cpp:101
+    vrank::check(vr_event_record(ev0, stream));
+    run((uint32_t)o.flag + 200);
+    vrank::check(vr_event_record(ev1, stream));
+    float ms = 0.f;
+    vrank::check(vr_event_elapsed_ms(ev0, ev1, &ms));
+    ranks.wait(stream);
+    printf("[%d] Running time: %lluns\n", rank, (unsigned long long)(ms * 1e6));
+  }
+  // nobody unmaps or frees while a peer may still be writing into it
+  vrank::check(vr_ipc_barrier(rank, world, o.instance.c_str(), ++generation));
+  vrank::check(vr_ipc_close_all(rank, world, bases));
+  vr_event_destroy(ev0);
+  vr_event_destroy(ev1);
+  vr_stream_destroy(stream);
+  vr_free(input);
+  vr_free(scratch);
+  return status;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) try {
@@ -148,6 +260,11 @@ int main(int argc, char **argv) try {
 
   if (o.dtype == "bf16") g_dtype = VR_DTYPE_BF16;
   else if (o.dtype != "f16") throw std::invalid_argument("dtype must be f16 or bf16");
+
+  if (o.rank >= 0) {
+    if (gather) throw std::invalid_argument("--rank runs all-reduce algos");
+    return run_as_rank(o, algo, nelems);
+  }
 
   vrank::VirtualRanks ranks(world, o.device);
   ranks.setDtype(g_dtype);

@@ -27,6 +27,9 @@
  *                        ParallelTransmit / BisectPTransmit ctors    parallel_transmit.hpp:36-60,
  *                                                                    bisect_transmit.hpp:427-482
  *   vr_rank_scratch_bytes <- interm_size = world * 8 MiB             main.cpp:241
+ *   vr_ipc_open_all   <- open_all_ipc_mems                           ipc_exchange.cpp:277-311
+ *                        (un_allgather over AF_UNIX sockets,         ipc_exchange.cpp:173-265)
+ *   vr_ipc_barrier    <- MPI_Barrier                                 main.cpp:101, 287
  */
 #ifndef VRANK_ALLREDUCE_H
 #define VRANK_ALLREDUCE_H
@@ -185,6 +188,24 @@ int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input
  * rank count, device and "wire_blocks_per_cu" setting. */
 int vr_rank_scratch_bytes(const vr_ctx *ctx, size_t *sink_bytes);
 
+/* ---- ranks in separate processes ------------------------------------------------ */
+
+/* open_all_ipc_mems: every one of `world` processes (one rank each, all on the
+ * same GPU or on GPUs with peer access) calls this with a pointer into a device
+ * allocation of its own (under 2 GiB).  The processes exchange IPC handles over
+ * AF_UNIX sockets named after `instance` and the rank (in $TMPDIR, else /tmp) and
+ * map each other's allocation: on return rank i's memory is at
+ * (char *)peer_bases[i] + offsets[i]; entry `rank` is `ptr` itself with offset 0.
+ * A peer that does not show up within 30 s (environment VRANK_IPC_TIMEOUT_MS
+ * overrides) ends the call with VR_ERR_TIMEOUT. */
+int vr_ipc_open_all(void *ptr, int rank, int world, void *peer_bases[], size_t offsets[],
+                    const char *instance);
+/* Unmaps what vr_ipc_open_all mapped (not the own entry). */
+int vr_ipc_close_all(int rank, int world, void *const peer_bases[]);
+/* Returns once all `world` processes of `instance` have called it with the same
+ * `generation` (a different number for every barrier of a run). */
+int vr_ipc_barrier(int rank, int world, const char *instance, int generation);
+
 /* No counterpart in the reference.  For callers that cannot allocate device
  * memory: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  A wire-transport vr_allreduce whose sinks live in a fixed
@@ -262,6 +283,15 @@ int vr_time_copy(vr_ctx *ctx, void *stream, void *dst, const void *src, size_t b
  *   VR_PROBE_WRITE writes dst, reads nothing */
 enum { VR_PROBE_COPY = 0, VR_PROBE_READ = 1, VR_PROBE_WRITE = 2 };
 int vr_stream_probe(vr_ctx *ctx, void *stream, int mode, void *dst, const void *src, size_t bytes);
+
+/* The all-reduce's own access shape as a yardstick: one launch of the direct
+ * all-reduce kernel with the adds removed, so that dsts[k] receives srcs[k]
+ * (`bytes_each` bytes, a multiple of 16 * nranks) for each of the context's
+ * nranks streams: the same grid, chunk walk, buffer addressing and cache policies
+ * as an out-of-place vr_allreduce of that size, N read streams and N write
+ * streams.  What this shape of traffic can reach without any arithmetic. */
+int vr_stream_probe_multi(vr_ctx *ctx, void *stream, void *const dsts[], const void *const srcs[],
+                          size_t bytes_each);
 
 /* Diagnostic: launches `blocks` work-groups and reports the XCD each one ran on
  * (ids_host[b]).  The direct kernels give work-group b to virtual rank b % N and

@@ -291,6 +291,26 @@ def test_config5_sweep_sizes(ctxs, oracle):
                 assert oracle.count_mismatch(got[r], got[0]) == 0, (algo, n, r)
 
 
+def test_multi_stream_copy_yardstick(ctxs, oracle):
+    """The all-reduce kernel with the adds removed copies stream k to stream k."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    for nranks, n in ((8, 8 * 8 * 1031), (8, 1 << 22), (4, 4 * 8 * 77), (2, 1 << 16)):
+        ins = H.make_inputs(oracle, nranks, n, 5600 + nranks)
+        src = H.RankBuffers(nranks, n)
+        src.upload(ins)
+        dst = H.RankBuffers(nranks, n)
+        dst.fill(0x11)
+        ctxs[nranks].stream_probe_multi(dst.ptrs, src.ptrs, n * 2)
+        ctxs[nranks].sync()
+        for a, b in zip(dst.download(), ins):
+            assert np.array_equal(a, b), (nranks, n)
+        src.free()
+        dst.free()
+    with pytest.raises(vr.VRError) as e:
+        ctxs[8].stream_probe_multi([16] * 8, [16] * 8, 8 * 16 + 16)
+    assert e.value.code == "UNEVEN"
+
+
 # ---- all-gather ---------------------------------------------------------------------------------
 
 def run_allgather(ctx, algo, ins, alias_own_slot=False):

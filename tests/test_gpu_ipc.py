@@ -1,0 +1,87 @@
+"""One process per rank on one GPU: every process owns its rank's input and
+scratch, the processes exchange IPC handles over AF_UNIX sockets and map each
+other's scratch (vr_ipc_open_all <- open_all_ipc_mems, ipc_exchange.cpp:277-311),
+and each launches its own rank's wires (vr_allreduce_rank).  The reference's own
+arrangement (mpirun -np N ./main), run through the CLI's --rank mode."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from tests import vr_helpers as H
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
+_runs = [0]
+
+
+def run_ranks(world, extra, per_rank=None, timeout=100):
+    """Start `world` rank processes, wait for all; returns [(returncode, output)]."""
+    _runs[0] += 1
+    instance = "g%d_%d" % (os.getpid(), _runs[0])
+    procs = []
+    for r in range(world):
+        cmd = [CLI, "-r", str(world), "--rank", str(r), "-i", instance] + extra + (per_rank(r) if per_rank else [])
+        procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    out = []
+    for p in procs:
+        try:
+            text, _ = p.communicate(timeout=timeout)
+        except subprocess.TimeoutExpired:
+            p.kill()                       # exactly the processes started here
+            text, _ = p.communicate()
+            text += "\n(killed after %d s)" % timeout
+        out.append((p.returncode, text))
+    return out
+
+
+@pytest.mark.parametrize("world,algo", [(2, "simple"), (4, "simple"), (2, "small"), (4, "bisect"),
+                                        (4, "parallel"), (2, "simple_ring"), (4, "small_pcie")])
+def test_fill_pattern_verify_across_processes(world, algo):
+    """main.cpp's -v flow in every rank process: fill_pattern inputs, the host sum
+    of allreduce.cpp:18-27 as the check."""
+    for n in (16384, 14336 * 4):
+        res = run_ranks(world, ["-v", "-n", str(n), "-a", algo])
+        for r, (rc, text) in enumerate(res):
+            assert rc == 0, (algo, n, r, text)
+            assert "match the host sum" in text and "Error Compare" not in text, (algo, n, r, text)
+
+
+@pytest.mark.parametrize("world,algo", [(2, "parallel"), (4, "parallel"), (4, "bisect"), (4, "simple_ring"),
+                                        (2, "small")])
+def test_seeded_inputs_match_the_oracle_across_processes(oracle, tmp_path, world, algo):
+    n = 1 << 20
+    seed = 9100 + world
+    res = run_ranks(world, ["-n", str(n), "-a", algo, "--seed", str(seed)],
+                    per_rank=lambda r: ["--dump", str(tmp_path / ("out%d.bin" % r))])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0, (algo, r, text)
+    ins = H.make_inputs(oracle, world, n, seed)          # the same generator, rank r seeded with seed + r
+    want = H.expected(oracle, algo, ins)
+    for r in range(world):
+        got = np.fromfile(tmp_path / ("out%d.bin" % r), np.uint16)
+        assert len(got) == n and oracle.count_mismatch(got, want) == 0, (algo, r)
+
+
+def test_timed_run_protocol_across_processes():
+    """Without -v: three warm-ups, a barrier, the timed run, one line per rank."""
+    res = run_ranks(4, ["-n", "1M", "-a", "simple"])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0 and "[%d] Running time: " % r in text, (r, text)
+
+
+def test_a_missing_rank_is_a_time_out_not_a_hang():
+    """Rank 1 of 2 never starts: rank 0 gives up waiting for its record."""
+    _runs[0] += 1
+    p = subprocess.Popen([CLI, "-r", "2", "--rank", "0", "-i", "lone%d" % os.getpid(), "-v", "-n", "4096",
+                          "-a", "simple"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                         env=dict(os.environ, VRANK_IPC_TIMEOUT_MS="2000"))
+    try:
+        text, _ = p.communicate(timeout=60)
+    except subprocess.TimeoutExpired:
+        p.kill()
+        text, _ = p.communicate()
+        pytest.fail("rank 0 did not give up: " + text)
+    assert p.returncode == 1 and "could not reach rank 1" in text, text
