@@ -22,15 +22,21 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (each scaled by the same counter's reading for a plain copy of known size);
-# see profiles/.  Keyed by workload name.
+# HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (each scaled by the same counter's reading for a plain copy of known size).
+# (workload, transport) -> (bytes, the summary under profiles/ that derives the
+# figure; a CPU test checks that the file states this very number).
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/direct_allreduce_bisect_8x32MiB_hbm_traffic.md
-    "cfg3": 536914021,
-    # profiles/direct_allgather_4x8MiB_kernel_trace.md
-    "cfg4": 167799218,
+    ("cfg3", "direct"): (536914021, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
+    ("cfg4", "direct"): (167799218, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
 }
+
+
+def measured_traffic(name, transport):
+    algo = WORKLOADS[name][1]
+    if transport == "default":
+        transport = "wire" if algo == "parallel" else "direct"
+    return MEASURED_TRAFFIC_BYTES.get((name, transport), (None, None))[0]
 
 # Element type of the run (--dtype): 0 = binary16, 1 = bfloat16.  Buffers are
 # 2-byte elements either way; only the adds and the generated bit patterns differ.
@@ -206,30 +212,47 @@ def cpu_leg(name, gpu_results, budget_s):
         mismatches[wname] = int(sum(o.count_mismatch_dt(DTYPE, g, want) for g in outs))
 
     host, fn = reference(name)
-    timing = {}
-    for label in ("all", "one"):
-        if label == "all":
-            env = os.environ.get("OMP_NUM_THREADS")
-            used = o.set_threads(int(env) if env else min(os.cpu_count() or 1, 64))
+    n, algo, *_ = WORKLOADS[name]
+    forms = [("device_order", fn)]
+    if not algo.startswith("allgather"):
+        # the reference's own host oracle: per element a chain over the ranks in rank
+        # order (allreduce.cpp:18-27), OpenMP over elements
+        if DTYPE == 0:
+            forms.append(("reference_rank_order", o.rank_order))
         else:
-            used = o.set_threads(1)
-        fn(host)                                          # warm-up, page faults
-        best, reps, t_start = 1e30, 0, time.perf_counter()
-        while True:
-            t0 = time.perf_counter()
-            fn(host)
-            dt = time.perf_counter() - t0
-            best, reps = min(best, dt), reps + 1
-            elapsed = time.perf_counter() - t_start
-            if (reps >= 5 and elapsed > budget_s / 4) or elapsed > budget_s / 2:
-                break
-        timing[label] = (algorithmic_bytes(name) / best / 1e9, used, reps, best)
-    gb_all, cores, reps, best = timing["all"]
-    baseline = {
-        "value": round(gb_all, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-        "sample": "%s full size, best of %d passes (%.1f ms); 1 thread: %.3f GB/s" % (
-            name, reps, best * 1e3, timing["one"][0]),
-    }
+            forms.append(("reference_rank_order", lambda ins: o.order_dt(DTYPE, oracle_lib.ORDER_RANK, ins)))
+    env = os.environ.get("OMP_NUM_THREADS")
+    all_threads = int(env) if env else min(os.cpu_count() or 1, 64)
+    share = budget_s / (2 * len(forms))
+    timing = {}
+    for form, f in forms:
+        for label, threads in (("all", all_threads), ("one", 1)):
+            used = o.set_threads(threads)
+            f(host)                                          # warm-up, page faults
+            best, reps, t_start = 1e30, 0, time.perf_counter()
+            while True:
+                t0 = time.perf_counter()
+                f(host)
+                dt = time.perf_counter() - t0
+                best, reps = min(best, dt), reps + 1
+                elapsed = time.perf_counter() - t_start
+                if (reps >= 5 and elapsed > share / 2) or elapsed > share:
+                    break
+            timing[(form, label)] = (algorithmic_bytes(name) / best / 1e9, used, reps, best)
+    o.set_threads(all_threads)
+    gb_all, cores, reps, best = timing[("device_order", "all")]
+    orders = {form: {"GBps_all_threads": round(timing[(form, "all")][0], 3),
+                     "GBps_one_thread": round(timing[(form, "one")][0], 3),
+                     "ms_all_threads": round(timing[(form, "all")][3] * 1e3, 2)}
+              for form, _ in forms}
+    text = "%s full size, best of %d passes (%.1f ms); 1 thread: %.3f GB/s" % (
+        name, reps, best * 1e3, timing[("device_order", "one")][0])
+    if "reference_rank_order" in orders:
+        text += "; the reference's rank-order host sum (allreduce.cpp:18-27): %.3f GB/s on %d threads, " \
+                "%.3f GB/s on 1" % (orders["reference_rank_order"]["GBps_all_threads"], cores,
+                                    orders["reference_rank_order"]["GBps_one_thread"])
+    baseline = {"value": round(gb_all, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": text, "orders": orders}
     return baseline, mismatches
 
 
@@ -410,7 +433,7 @@ def main():
         "bit_exact_vs_oracle": None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "traffic": measured_traffic(name, args.transport),
                      "kernel_us_avg": round(k_avg * 1e3, 3),
                      "kernel_us_p50": round(float(np.median(kms)) * 1e3, 3)},
     }
@@ -442,18 +465,30 @@ def main():
             gpu_results["cfg2"] = [b.download(np.uint16, WORKLOADS["cfg2"][2]) for b in s2[0][0]]
         time_kernels(binding, c2, "cfg2", s2, 50)
         lat = time_kernels(binding, c2, "cfg2", s2, args.latency_iters) * 1e3
-        p50 = float(np.percentile(lat, 50))
+        raw50, raw99 = float(np.percentile(lat, 50)), float(np.percentile(lat, 99))
+        # what an event pair costs with nothing between its two records
+        empty = binding.EventTimer(200)
+        for k in range(200):
+            empty.start(k)
+            empty.stop(k)
+        c2.sync()
+        overhead = float(np.median(empty.elapsed_ms())) * 1e3
+        empty.close()
         back_to_back = time_kernels(binding, c2, "cfg2", s2, args.latency_iters, group=20) * 1e3
+        p50 = float(np.median(back_to_back))
         result["latency_1MiB_per_rank"] = {
             "workload": describe("cfg2") + ", in place", "iters": args.latency_iters,
-            "p50_us": round(p50, 3), "p99_us": round(float(np.percentile(lat, 99)), 3),
-            "min_us": round(float(lat.min()), 3),
-            "back_to_back_us": round(float(np.median(back_to_back)), 3),
+            "p50_us": round(p50, 3),
+            "p99_us": round(float(np.percentile(back_to_back, 99)), 3),
+            "single_launch_events": {"p50_us": round(raw50, 3), "p99_us": round(raw99, 3),
+                                     "min_us": round(float(lat.min()), 3),
+                                     "event_pair_overhead_us": round(overhead, 3),
+                                     "p50_minus_overhead_us": round(raw50 - overhead, 3)},
             "bit_exact_vs_oracle": None,
             "GBps_at_p50": round(algorithmic_bytes("cfg2") / (p50 * 1e-6) / 1e9, 1),
-            "note": "p50/p99: one HIP event pair per launch, which includes ~2.7 us of event "
-                    "overhead (a kernel trace shows p50 4.2-4.5 us); back_to_back_us: 20 launches per "
-                    "event pair, per launch; buffers are cache-resident"}
+            "note": "p50_us / p99_us: per launch, from event pairs that bracket 20 back-to-back launches "
+                    "(%d groups); single_launch_events: one event pair per launch, which adds the "
+                    "measured event_pair_overhead_us; buffers are cache-resident" % len(back_to_back)}
         result["hbm_ceilings"] = hbm_ceilings(binding, ctx)
         if sets[0][1] is not None and not algo.startswith("allgather"):
             # the same kernel, grid and policies without the adds, on the same buffer sets

@@ -187,10 +187,14 @@ struct WireLL {
                          VR_AGENT);
     }
   }
+  // watch_first: the message is expected to be still on its way, so start by
+  // watching its last flag word instead of reading the whole message in vain.
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
-                                              uint32_t flag, uint32_t lane, Spin &spin) {
+                                              uint32_t flag, uint32_t lane, Spin &spin,
+                                              bool watch_first = false) {
     if (spin.dead) return false;
     const char *const one[1] = {slot};
+    if (watch_first && !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     uint32_t polls = 0;
     for (;;) {
       bool ok = true;
@@ -290,10 +294,14 @@ struct WireLL16 {
       __builtin_amdgcn_raw_buffer_store_b128(msg, rs, (u * 64u + lane) * 16u, 0, kAuxAgent);
     }
   }
+  // watch_first: the message is expected to be still on its way, so start by
+  // watching its last flag word instead of reading the whole message in vain.
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
-                                              uint32_t flag, uint32_t lane, Spin &spin) {
+                                              uint32_t flag, uint32_t lane, Spin &spin,
+                                              bool watch_first = false) {
     if (spin.dead) return false;
     const char *const one[1] = {slot};
+    if (watch_first && !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     const __amdgpu_buffer_rsrc_t rs = rsrc(slot);
     uint32_t polls = 0;
     for (;;) {
@@ -412,10 +420,14 @@ struct WireRt128 {
     v.d[u][1] = l == 7u ? back : y;                                      // restoreData
     return ((l & 7u) != 7u) | (y == flag);
   }
+  // watch_first: the message is expected to be still on its way, so start by
+  // watching its last flag word instead of reading the whole message in vain.
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
-                                              uint32_t flag, uint32_t lane, Spin &spin) {
+                                              uint32_t flag, uint32_t lane, Spin &spin,
+                                              bool watch_first = false) {
     if (spin.dead) return false;
     const char *const one[1] = {slot};
+    if (watch_first && !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     uint32_t polls = 0;
     for (;;) {
       uint64_t raw[U];
@@ -529,10 +541,14 @@ struct WireRt256 {
     v.d[u][3] = l == 3u ? b3 : l == 7u ? b7 : l == 11u ? b11 : msg.w;
     return ((l & 3u) != 3u) | (msg.w == flag);
   }
+  // watch_first: the message is expected to be still on its way, so start by
+  // watching its last flag word instead of reading the whole message in vain.
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
-                                              uint32_t flag, uint32_t lane, Spin &spin) {
+                                              uint32_t flag, uint32_t lane, Spin &spin,
+                                              bool watch_first = false) {
     if (spin.dead) return false;
     const char *const one[1] = {slot};
+    if (watch_first && !await_last_flags<1>(one, kSlotBytes, flag, lane, spin)) return false;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot, kSlotBytes);
     uint32_t polls = 0;
     for (;;) {
@@ -618,7 +634,8 @@ struct WireFlag {
     if (lane == 0) __hip_atomic_store(flagword, flag, __ATOMIC_RELAXED, VR_AGENT);
   }
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *flagword, Reg &v,
-                                              uint32_t flag, uint32_t lane, Spin &spin) {
+                                              uint32_t flag, uint32_t lane, Spin &spin,
+                                              bool /*watch_first*/ = false) {
     if (spin.dead) return false;
     uint32_t polls = 0;
     // All lanes read the same word, so the loop condition is wave-uniform.
@@ -725,7 +742,7 @@ __global__ __launch_bounds__(256) void k_wire_parallel(WireArgs a) {
       if (off + kAhead * stride < chunk) scatter(off + kAhead * stride, t + kAhead);
       typename W::Reg v;
       const uint32_t slot = wl::parallel_slot(x_id, y, s);
-      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin, true);   // the owner is still reducing
       W::store(dst + off, left, lane, v, nt);
     }
   } else {
@@ -1010,7 +1027,7 @@ __global__ __launch_bounds__(256) void k_wire_bisect(WireArgs a) {
     typename W::Reg v = cur;
     if ((int)y != l) {
       const uint32_t slot = wl::bisect_close_slot(wg, y, s);
-      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin);
+      W::recv(sk.gath(r, slot), sk.gflag(r, slot), v, flag, lane, spin, true);   // the owner is still reducing
     } else {
       const char *ms[B - 1];
       const uint32_t *mf[B - 1];
@@ -1035,7 +1052,7 @@ __global__ __launch_bounds__(256) void k_wire_bisect(WireArgs a) {
     W::store(dst + close_off + off, left, lane, v, nt);
     {                                                 // pollFarGatherOutput
       typename W::Reg m;
-      W::recv(sk.gath(r, far), sk.gflag(r, far), m, flag, lane, spin);
+      W::recv(sk.gath(r, far), sk.gflag(r, far), m, flag, lane, spin, true);      // the pair forwards last
       W::store(dst + far_off + off, left, lane, m, nt);
     }
     cur = nxt;

@@ -22,3 +22,17 @@ def test_algorithmic_bytes_match_the_metric_definition():
     assert bench.WORKLOADS["cfg3"][:3] == (8, "bisect", 16777216)
     assert bench.WORKLOADS["cfg2"][:3] == (8, "small", 524288)
     assert bench.WORKLOADS["cfg4"][:3] == (4, "allgather_simple", 4194304)
+
+
+def test_measured_traffic_constants_are_the_numbers_in_the_profiles():
+    """roofline.traffic is a constant copied from a counter run: the summary under
+    profiles/ it names must state exactly that number."""
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.MEASURED_TRAFFIC_BYTES
+    for (workload, transport), (nbytes, fname) in bench.MEASURED_TRAFFIC_BYTES.items():
+        assert workload in bench.WORKLOADS and transport in ("direct", "wire")
+        text = open(os.path.join(ROOT, "profiles", fname)).read()
+        assert "{:,} B".format(nbytes) in text, (workload, transport, nbytes, fname)
+    assert bench.measured_traffic("cfg3", "default") == bench.MEASURED_TRAFFIC_BYTES[("cfg3", "direct")][0]
+    assert bench.measured_traffic("cfg3", "wire") == bench.MEASURED_TRAFFIC_BYTES.get(("cfg3", "wire"), (None,))[0]

@@ -255,6 +255,22 @@ def test_fenced_flag_word_format(oracle, algo):
     ctx.close()
 
 
+@pytest.mark.parametrize("algo", ["simple", "parallel", "bisect", "simple_ring", "simple_pcie"])
+def test_eight_byte_messages_for_the_128_byte_families(oracle, algo):
+    """wire_fenced=2: the Rt64_128 families travel as self-validating 8-byte messages
+    (payload dword + flag), which assume nothing beyond 8-byte store atomicity."""
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_fenced=2)
+    for n in (64, 64 * 129, 1 << 19):
+        ins = H.make_inputs(oracle, 8, n, 6500 + n)
+        for inplace in (True, False):
+            got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, inplace=inplace)
+            H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+    with pytest.raises(vr.VRError):
+        ctx.set_tuning(wire_fenced=3)
+    ctx.close()
+
+
 @pytest.mark.parametrize("cooperative", [0, 1])
 def test_plain_and_cooperative_launch(oracle, cooperative):
     """By default the launch is plain when the occupancy query proves the grid
