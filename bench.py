@@ -29,6 +29,8 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("cfg3", "direct"): (536914021, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
     ("cfg4", "direct"): (167799218, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
+    ("cfg5_32MiB", "wire"): (1551376119, "wire_allreduce_parallel_8x32MiB.md"),
+    ("cfg3", "wire"): (1562205164, "wire_allreduce_bisect_8x32MiB.md"),
 }
 
 
@@ -293,20 +295,32 @@ def sweep(vr, binding, args):
     # The fastest protocol per size; a protocol only takes over when it is more
     # than 3 % faster than the incumbent, so that timer noise between kernels
     # that perform alike does not read as a crossover.
-    best = []
-    for i, S in enumerate(sizes):
-        fastest = min(curves, key=lambda k: curves[k][i]["us"])
-        if best and curves[best[-1]][i]["us"] <= 1.03 * curves[fastest][i]["us"]:
-            fastest = best[-1]
-        best.append(fastest)
-    crossovers = [{"bytes_per_rank": sizes[i], "from": best[i - 1], "to": best[i]}
-                  for i in range(1, len(sizes)) if best[i] != best[i - 1]]
+    def fastest_of(keys):
+        best = []
+        for i in range(len(sizes)):
+            fastest = min(keys, key=lambda k: curves[k][i]["us"])
+            if best and curves[best[-1]][i]["us"] <= 1.03 * curves[fastest][i]["us"]:
+                fastest = best[-1]
+            best.append(fastest)
+        cross = [{"bytes_per_rank": sizes[i], "from": best[i - 1], "to": best[i]}
+                 for i in range(1, len(sizes)) if best[i] != best[i - 1]]
+        return best, cross
+
+    best, crossovers = fastest_of(list(curves))
+    # The same question inside the message-passing family, where the four protocols
+    # are different kernels with different wire formats and flows (the form that
+    # would run across GPUs): small = 8-byte messages, simple / parallel = 128 / 256-byte
+    # messages over ParallelTransmit, bisect = pair exchange + 4-way exchange.
+    wire_keys = [k for k in ("small@wire", "simple@wire", "bisect@wire", "parallel") if k in curves]
+    wire_best, wire_cross = fastest_of(wire_keys) if len(wire_keys) > 1 else ([], [])
     print(json.dumps({"metric": "allreduce_GBps_vs_size_8vrank_fp16", "unit": "GB/s",
                       "note": "in place on one buffer set: sizes up to 16 MiB/rank are served by "
                               "the caches, 64 MiB/rank and above stream from HBM; times are HIP-event "
                               "times of single launches (~2 us of event overhead included)",
                       "curves": curves, "fastest": dict(zip(map(str, sizes), best)),
-                      "crossovers": crossovers}))
+                      "crossovers": crossovers,
+                      "fastest_message_passing": dict(zip(map(str, sizes), wire_best)),
+                      "crossovers_message_passing": wire_cross}))
 
 
 def main():

@@ -70,6 +70,7 @@ def lib():
         "vr_ctx_reserve_wire": (i, [vp]),
         "vr_ctx_nranks": (i, [vp]),
         "vr_allreduce_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
+        "vr_allgather_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
         "vr_rank_scratch_bytes": (i, [vp, C.POINTER(sz)]),
         "vr_allreduce_static": (i, [vp, vp, i, vpp, vpp, sz]),
         "vr_ctx_set_dtype": (i, [vp, i]),
@@ -274,6 +275,16 @@ class VirtualRanks:
                                        C.c_void_p(int(scatter)), C.c_void_p(int(gather)),
                                        _table(peers0), _table(peers1), sink_bytes, nelems,
                                        C.byref(seq)))
+        return seq.value
+
+    def allgather_rank(self, algo, rank, inp, out, scatter, gather, peers0, peers1, sink_bytes, nelems,
+                       seq_no, stream=None):
+        """One rank of the ring all-gather against caller-owned sinks."""
+        seq = C.c_uint32(seq_no)
+        _check(lib().vr_allgather_rank(self._h, stream, algo_id(algo), rank, C.c_void_p(int(inp)),
+                                       C.c_void_p(int(out)), C.c_void_p(int(scatter)),
+                                       C.c_void_p(int(gather)), _table(peers0), _table(peers1),
+                                       sink_bytes, nelems, C.byref(seq)))
         return seq.value
 
     def allreduce_static(self, algo, bufs, nelems, outs=None, stream=None):

@@ -863,6 +863,32 @@ extern "C" int vr_allreduce_static(vr_ctx *ctx, void *stream, int algo, void *co
                      0, &used, wlch);
 }
 
+// Caller-owned sinks of a one-rank launch: the rank's own pair and its peers'.
+static int rank_sinks(const vr_ctx *ctx, int rank, void *scatter_buf, void *gather_buf,
+                      void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes, WireSinks *k) {
+  const int N = ctx->nranks;
+  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!scatter_buf || !gather_buf || !peer_buf0 || !peer_buf1)
+    return fail(VR_ERR_INVALID, "null scratch pointer");
+  const uint32_t wpr_max = wire_wpr_max(ctx);
+  const wl::Layout l = wl::layout_for(N, wpr_max, true);
+  if (sink_bytes < l.sink_bytes)
+    return fail(VR_ERR_INVALID, "sinks hold " + std::to_string(sink_bytes) + " bytes, this context needs " +
+                                    std::to_string(l.sink_bytes) + " (vr_rank_scratch_bytes)");
+  *k = WireSinks();
+  k->layout = l;
+  k->wpr_max = wpr_max;
+  k->simple_ok = true;
+  for (int r = 0; r < N; ++r) {
+    k->scatter[r] = r == rank ? scatter_buf : peer_buf0[r];
+    k->gather[r] = r == rank ? gather_buf : peer_buf1[r];
+    if (!k->scatter[r] || !k->gather[r]) return fail(VR_ERR_INVALID, "null peer sink for rank " + std::to_string(r));
+    if ((uintptr_t)k->scatter[r] % 16 || (uintptr_t)k->gather[r] % 16)
+      return fail(VR_ERR_UNALIGNED, "sinks must be 16-byte aligned");
+  }
+  return VR_OK;
+}
+
 // One rank of an all-reduce, the form the reference constructs per process
 // (allreduce.hpp:18-28, parallel_transmit.hpp:36-60, bisect_transmit.hpp:427-482).
 extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
@@ -875,8 +901,6 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
   const int N = ctx->nranks;
   if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
   if (!seq_no) return fail(VR_ERR_INVALID, "a one-rank launch needs the caller's sequence number");
-  if (!scatter_buf || !gather_buf || !peer_buf0 || !peer_buf1)
-    return fail(VR_ERR_INVALID, "null scratch pointer");
   if (!output) output = input;
   // calcWorkSize sees this rank's pointers only (allreduce.hpp:108-122).
   const void *table[VR_MAX_RANKS];
@@ -887,22 +911,8 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
   if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
   if (ranges_partially_overlap(output, input, nelems * 2))
     return fail(VR_ERR_OVERLAP, "output partially overlaps input");
-  const uint32_t wpr_max = wire_wpr_max(ctx);
-  const wl::Layout l = wl::layout_for(N, wpr_max, true);
-  if (sink_bytes < l.sink_bytes)
-    return fail(VR_ERR_INVALID, "sinks hold " + std::to_string(sink_bytes) + " bytes, this context needs " +
-                                    std::to_string(l.sink_bytes) + " (vr_rank_scratch_bytes)");
   WireSinks k;
-  k.layout = l;
-  k.wpr_max = wpr_max;
-  k.simple_ok = true;
-  for (int r = 0; r < N; ++r) {
-    k.scatter[r] = r == rank ? scatter_buf : peer_buf0[r];
-    k.gather[r] = r == rank ? gather_buf : peer_buf1[r];
-    if (!k.scatter[r] || !k.gather[r]) return fail(VR_ERR_INVALID, "null peer sink for rank " + std::to_string(r));
-    if ((uintptr_t)k.scatter[r] % 16 || (uintptr_t)k.gather[r] % 16)
-      return fail(VR_ERR_UNALIGNED, "sinks must be 16-byte aligned");
-  }
+  if (int rc = rank_sinks(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
   PtrTable in, out;
   memset(&in, 0, sizeof in);
   memset(&out, 0, sizeof out);
@@ -920,6 +930,49 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
   if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, chunk_elems * 2, vec_halves, &seq, 0,
                            &used, wlch))
     return rc;
+  *seq_no = seq + (used > geom.steps ? used : geom.steps);
+  if (*seq_no == 0) *seq_no = 1;
+  return VR_OK;
+}
+
+// One rank of the ring all-gather (AllGather(input, output, nelems, rank, seqNo, scatterBuf,
+// gatherBuf, peerBuf0, peerBuf1), allgather.hpp:19-29, 58-70).
+extern "C" int vr_allgather_rank(vr_ctx *ctx, void *stream, int algo, int rank, const void *input,
+                                 void *output, void *scatter_buf, void *gather_buf,
+                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
+                                 size_t nelems, uint32_t *seq_no) {
+  if (int rc = use_device(ctx)) return rc;
+  const AlgoInfo *a = algo_info(algo);
+  if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
+  const int N = ctx->nranks;
+  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!seq_no) return fail(VR_ERR_INVALID, "a one-rank launch needs the caller's sequence number");
+  // allgather.hpp:104-117 for this rank's pointers
+  const void *ins[VR_MAX_RANKS];
+  void *outs[VR_MAX_RANKS];
+  for (int r = 0; r < N; ++r) {
+    ins[r] = input;
+    outs[r] = output;
+  }
+  if (int rc = vr_check_allgather(algo, N, ins, outs, nelems, nullptr)) return rc;
+  const size_t bytes = nelems * 2;
+  const char *own_slot = static_cast<const char *>(output) + (size_t)rank * bytes;
+  const uintptr_t x = (uintptr_t)input, y = (uintptr_t)output;
+  if (x < y + bytes * N && y < x + bytes && (const void *)own_slot != input)
+    return fail(VR_ERR_OVERLAP, "input overlaps output other than as its own slot");
+  WireSinks k;
+  if (int rc = rank_sinks(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
+  PtrTable in, out;
+  memset(&in, 0, sizeof in);
+  memset(&out, 0, sizeof out);
+  in.p[rank] = const_cast<void *>(input);
+  out.p[rank] = output;
+  vr_geometry geom;
+  if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
+  const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};
+  uint32_t seq = *seq_no, used = 0;
+  // messages are 16 bytes, so every pointer and the slice allow 16-byte accesses
+  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, bytes, 8, &seq, 0, &used, wlch)) return rc;
   *seq_no = seq + (used > geom.steps ? used : geom.steps);
   if (*seq_no == 0) *seq_no = 1;
   return VR_OK;

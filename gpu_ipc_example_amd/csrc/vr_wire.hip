@@ -1114,17 +1114,22 @@ hipError_t wire_static_scratch(int device, void **ptr, size_t *bytes) {
 template <typename W>
 static const void *flow_kernel(WireFlow flow, int nranks) {
   const void *fn = nullptr;
+  // World sizes the reference's dispatchers instantiate: 2, 4, 8 for the flat and
+  // ring transmits (allreduce.cpp:854-881), 4, 8, 16 for bisect (l.1003-1030).
 #define VR_PICK(NN)                                                                         \
   case NN:                                                                                  \
-    switch (flow) {                                                                         \
-      case WIRE_PARALLEL: fn = reinterpret_cast<const void *>(&k_wire_parallel<NN, W>); break;   \
-      case WIRE_SEQUENTIAL: fn = reinterpret_cast<const void *>(&k_wire_sequential<NN, W>); break; \
-      case WIRE_SIMPLE: fn = reinterpret_cast<const void *>(&k_wire_simple<NN, W>); break;         \
-      case WIRE_RING: fn = reinterpret_cast<const void *>(&k_wire_ring<NN, W>); break;           \
-      case WIRE_ALLGATHER: fn = reinterpret_cast<const void *>(&k_wire_allgather<NN, W>); break;  \
-      case WIRE_BISECT:                                                                     \
-        if constexpr (NN >= 4) fn = reinterpret_cast<const void *>(&k_wire_bisect<NN, W>);  \
-        break;                                                                              \
+    if constexpr (NN <= 8) {                                                                \
+      switch (flow) {                                                                       \
+        case WIRE_PARALLEL: fn = reinterpret_cast<const void *>(&k_wire_parallel<NN, W>); break;   \
+        case WIRE_SEQUENTIAL: fn = reinterpret_cast<const void *>(&k_wire_sequential<NN, W>); break; \
+        case WIRE_SIMPLE: fn = reinterpret_cast<const void *>(&k_wire_simple<NN, W>); break;         \
+        case WIRE_RING: fn = reinterpret_cast<const void *>(&k_wire_ring<NN, W>); break;           \
+        case WIRE_ALLGATHER: fn = reinterpret_cast<const void *>(&k_wire_allgather<NN, W>); break;  \
+        default: break;                                                                     \
+      }                                                                                     \
+    }                                                                                       \
+    if constexpr (NN >= 4) {                                                                \
+      if (flow == WIRE_BISECT) fn = reinterpret_cast<const void *>(&k_wire_bisect<NN, W>);  \
     }                                                                                       \
     break;
   switch (nranks) {

@@ -26,6 +26,7 @@
  *                        peerBuf0[], peerBuf1[]) + queue.submit      allreduce.hpp:18-28, 64-74
  *                        ParallelTransmit / BisectPTransmit ctors    parallel_transmit.hpp:36-60,
  *                                                                    bisect_transmit.hpp:427-482
+ *   vr_allgather_rank <- AllGather(input, output, nelems, rank, seqNo, ...)  allgather.hpp:19-29, 58-70
  *   vr_rank_scratch_bytes <- interm_size = world * 8 MiB             main.cpp:241
  *   vr_ipc_open_all   <- open_all_ipc_mems                           ipc_exchange.cpp:277-311
  *                        (un_allgather over AF_UNIX sockets,         ipc_exchange.cpp:173-265)
@@ -182,6 +183,12 @@ int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void 
  * library neither allocates nor clears anything here.  vr_ctx_check(ctx, stream)
  * reports a time-out of this context's launches. */
 int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
+                      void *scatter_buf, void *gather_buf, void *const peer_buf0[],
+                      void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+/* One rank of the ring all-gather, same contract (AllGather(input, output, nelems,
+ * rank, seqNo, scatterBuf, gatherBuf, peerBuf0, peerBuf1), allgather.hpp:19-29):
+ * output holds nranks * nelems elements; output + rank * nelems may be input. */
+int vr_allgather_rank(vr_ctx *ctx, void *stream, int algo, int rank, const void *input, void *output,
                       void *scatter_buf, void *gather_buf, void *const peer_buf0[],
                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
 /* Bytes a scatter sink (and equally a gather sink) must hold for this context's

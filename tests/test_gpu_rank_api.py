@@ -104,6 +104,43 @@ def test_rank_launches_match_the_oracle(ranks, oracle, nranks, algo):
             H.assert_all_ranks_equal(oracle, got, want, "%s N=%d n=%d" % (algo, nranks, n))
 
 
+@pytest.mark.parametrize("nranks", [2, 4])
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_rank_allgather(ranks, oracle, nranks, algo):
+    """The ring all-gather as one launch per rank, also with a rank's input aliased to
+    its own output slot (sequential_transmit.hpp:496-497)."""
+    R = ranks[nranks]
+    R.zero()
+    seq = 1
+    s0 = [b.ptr for b in R.scatter]
+    s1 = [b.ptr for b in R.gather]
+    for n in (8, 8 * 1237, 1 << 18):
+        ins = H.make_inputs(oracle, nranks, n, 8500 + n)
+        want = oracle.allgather(ins)
+        for alias in (False, True):
+            outs = [DeviceBuffer(nranks * n * 2) for _ in range(nranks)]
+            srcs = []
+            for r in range(nranks):
+                outs[r].fill(0x01)
+                if alias:
+                    outs[r].upload(ins[r], r * n * 2)
+                else:
+                    srcs.append(DeviceBuffer(n * 2))
+                    srcs[r].upload(ins[r])
+            nxt = seq
+            for r in range(nranks):
+                inp = outs[r].ptr + r * n * 2 if alias else srcs[r].ptr
+                nxt = R.ctx[r].allgather_rank(algo, r, inp, outs[r].ptr, s0[r], s1[r], s0, s1, R.sink_bytes, n,
+                                              seq, stream=R.handle(r))
+            for r in range(nranks):
+                R.ctx[r].check(R.handle(r))
+            seq = nxt
+            for r in range(nranks):
+                assert np.array_equal(outs[r].download(np.uint16, nranks * n), want), (algo, n, r, alias)
+            for b in outs + srcs:
+                b.free()
+
+
 LAYOUTS = {
     # algo: (oracle wire kind, payload bytes a wave moves per step, reference messages per wave and step)
     "small": (WIRE_RT64, 1024, 16),
