@@ -239,6 +239,8 @@ struct WireSinks {
   wl::Layout layout = {};
   uint32_t wpr_max = 0;        // wires per rank the sinks hold
   bool simple_ok = false;      // room for SimpleTransmit's sender sections
+  void *region = nullptr;      // library-owned sinks lie back to back in one region of
+  size_t region_bytes = 0;     // this many bytes (cleared with one launch)
 };
 
 // What earlier launches left in a set of sinks.
@@ -303,6 +305,8 @@ static void sinks_at(WireSinks *k, int nranks, char *base, const wl::Layout &l, 
   k->layout = l;
   k->wpr_max = wpr_max;
   k->simple_ok = simple_ok;
+  k->region = base;
+  k->region_bytes = (size_t)nranks * l.rank_bytes;
 }
 
 extern "C" int vr_ctx_reserve_wire(vr_ctx *c) {
@@ -333,6 +337,10 @@ extern "C" int vr_rank_scratch_bytes(const vr_ctx *c, size_t *sink_bytes) {
 
 // Forget every flag ever written (asynchronous, ordered on `s`).
 static int wire_clear(const WireSinks &k, int nranks, hipStream_t s) {
+  if (k.region) {
+    const hipError_t e = launch_wire_clear(s, k.region, k.region_bytes);
+    return e == hipSuccess ? VR_OK : fail_hip(e, "launch_wire_clear");
+  }
   for (int r = 0; r < nranks; ++r) {
     hipError_t e = launch_wire_clear(s, k.scatter[r], k.layout.sink_bytes);
     if (e == hipSuccess) e = launch_wire_clear(s, k.gather[r], k.layout.sink_bytes);
@@ -919,10 +927,13 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
   in.p[rank] = input;
   out.p[rank] = output;
   const size_t chunk_elems = work / 2;
-  const bool align16 = (uintptr_t)input % 16 == 0 && (uintptr_t)output % 16 == 0;
-  // Every rank must pick the same message shape; only the fenced format depends on
-  // the access width, and there the caller's buffers decide it for all ranks.
-  const int vec_halves = (align16 && chunk_elems % 8 == 0) ? 8 : 4;
+  // Every rank must pick the same message shape, so the access width may depend on
+  // nothing but the element count: 16-byte accesses whenever the chunk is a
+  // multiple of 16 bytes, and then this rank's buffers must allow them.
+  const int vec_halves = chunk_elems % 8 == 0 ? 8 : 4;
+  if (vec_halves == 8 && ((uintptr_t)input % 16 || (uintptr_t)output % 16))
+    return fail(VR_ERR_UNALIGNED, "one-rank launches move a chunk that is a multiple of 16 bytes with 16-byte "
+                                  "accesses on every rank: input and output must be 16-byte aligned");
   vr_geometry geom;
   if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
   const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};

@@ -31,6 +31,9 @@
 // another wave has given up) a wave records a time-out in the status word and
 // runs to completion without waiting again, so the grid always drains.
 
+#include <mutex>
+#include <unordered_map>
+
 #include "vr_internal.h"
 
 namespace vr {
@@ -1181,7 +1184,24 @@ hipError_t wire_blocks_per_cu(WireFlow flow, WireFormat fmt, int vec_halves, int
                               uint32_t block_threads, DType dtype, int *per_cu) {
   const void *fn = wire_kernel(flow, fmt, vec_halves, nranks, dtype);
   if (!fn) return hipErrorInvalidValue;
-  return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, (int)block_threads, 0);
+  // The answer is a property of the kernel (every launch uses the same block size
+  // and no dynamic LDS): ask the runtime once per kernel, not once per launch.
+  static std::mutex lock;
+  static std::unordered_map<const void *, int> known;
+  {
+    std::lock_guard<std::mutex> hold(lock);
+    const auto it = known.find(fn);
+    if (it != known.end()) {
+      *per_cu = it->second;
+      return hipSuccess;
+    }
+  }
+  const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, (int)block_threads, 0);
+  if (e == hipSuccess) {
+    std::lock_guard<std::mutex> hold(lock);
+    known[fn] = *per_cu;
+  }
+  return e;
 }
 
 // cooperative: a cooperative launch makes the runtime check co-residency once

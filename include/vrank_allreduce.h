@@ -179,7 +179,10 @@ int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void 
  *              16-byte aligned, and was zeroed once before the first launch.
  *   seq_no   : in/out; must be the same on every rank and only ever grow; a
  *              change of algo needs freshly zeroed sinks.
- * Same validation and error codes as vr_allreduce for this rank's pointers.  The
+ * Same validation and error codes as vr_allreduce for this rank's pointers; in
+ * addition, when nelems / nranks is a multiple of 8 elements the chunk travels
+ * with 16-byte accesses on every rank, and input and output must be 16-byte
+ * aligned (VR_ERR_UNALIGNED otherwise).  The
  * library neither allocates nor clears anything here.  vr_ctx_check(ctx, stream)
  * reports a time-out of this context's launches. */
 int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,

@@ -1,6 +1,7 @@
 """Randomised parity sweep: random world size, protocol, transport, element
 count, alignment, in/out-of-place choice and launch knobs (cache policy, unroll,
-residency, segment length, scatter run-ahead), each checked bit for bit against
+residency, segment length, scatter run-ahead, wire format variant, streaming I/O),
+each checked bit for bit against
 the oracle.  Seeds are fixed, so a failure names a reproducible case."""
 import random
 
@@ -35,7 +36,9 @@ def test_random_cases(oracle, seed):
             grid = (rng.choice((1, 2, 3, 7, 16, 33, 64)), rng.choice((4, 8, 12, 32, 64)), rng.choice((16, 32)))
         knobs = dict(nt_load=rng.choice((-1, 0, 1)), nt_store=rng.choice((-1, 0, 1, 2)),
                      unroll=rng.choice((-1, 1, 2, 4)), segment_kib=rng.choice((-1, -1, 4, 64)),
-                     waves_per_cu=rng.choice((-1, 1, 4, 32)), wire_ahead=rng.choice((-1, 1, 3, 6)))
+                     waves_per_cu=rng.choice((-1, 1, 4, 32)), wire_ahead=rng.choice((-1, 1, 3, 6)),
+                     wire_fenced=rng.choice((-1, -1, 0, 1, 2)), wire_stream_io=rng.choice((-1, 0, 1)),
+                     wire_msg16=rng.choice((-1, 0, 1)), wire_cooperative=rng.choice((-1, -1, 1)))
         ctxs[nranks].set_tuning(**knobs)
         ins = H.make_inputs(oracle, nranks, n, 10_000 * seed + 37 * case,
                             p1=rng.choice((0.02, 1.0, 30.0, 3000.0)))

@@ -213,7 +213,35 @@ def test_rank_call_validates_like_the_constructor(ranks):
     with pytest.raises(vr.VRError) as e:
         c.allreduce_rank("simple", 0, buf.ptr, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 0)
     assert e.value.code == "INVALID"
+    # a chunk of 16-byte multiples travels with 16-byte accesses on every rank
+    with pytest.raises(vr.VRError) as e:
+        c.allreduce_rank("simple", 0, buf.ptr + 8, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 1)
+    assert e.value.code == "UNALIGNED" and "16-byte" in e.value.detail
     buf.free()
+
+
+@pytest.mark.parametrize("algo", ["simple", "parallel", "small", "bisect"])
+def test_eight_byte_granular_chunks_through_the_rank_calls(ranks, oracle, algo):
+    """Chunks that are only a multiple of 8 bytes (and buffers that are only 8-byte
+    aligned) take the 8-byte access path on every rank."""
+    R = ranks[4]
+    R.zero()
+    seq = 1
+    for n, offset in ((4 * 4 * 1001, 0), (4 * 4 * 33, 8)):
+        ins = H.make_inputs(oracle, 4, n, 8600 + n)
+        src = H.RankBuffers(4, n, offset)
+        src.upload(ins)
+        s0 = [b.ptr for b in R.scatter]
+        s1 = [b.ptr for b in R.gather]
+        nxt = seq
+        for r in range(4):
+            nxt = R.ctx[r].allreduce_rank(algo, r, src.ptrs[r], s0[r], s1[r], s0, s1, R.sink_bytes, n, seq,
+                                          stream=R.handle(r))
+        for r in range(4):
+            R.ctx[r].check(R.handle(r))
+        seq = nxt
+        H.assert_all_ranks_equal(oracle, src.download(), H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+        src.free()
 
 
 def test_a_rank_without_peers_times_out_and_drains(oracle):
