@@ -71,6 +71,7 @@ def lib():
         "vr_ctx_nranks": (i, [vp]),
         "vr_allreduce_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
         "vr_allgather_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
+        "vr_allreduce_rank_grid": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, u32, u32, u32, u32]),
         "vr_rank_scratch_bytes": (i, [vp, C.POINTER(sz)]),
         "vr_allreduce_static": (i, [vp, vp, i, vpp, vpp, sz]),
         "vr_ctx_set_dtype": (i, [vp, i]),
@@ -276,6 +277,14 @@ class VirtualRanks:
                                        _table(peers0), _table(peers1), sink_bytes, nelems,
                                        C.byref(seq)))
         return seq.value
+
+    def allreduce_rank_grid(self, algo, rank, inp, scatter, gather, peers0, peers1, sink_bytes, nelems,
+                            seq_no, groups, subgroups, simd=16, out=None, stream=None):
+        _check(lib().vr_allreduce_rank_grid(self._h, stream, algo_id(algo), rank, C.c_void_p(int(inp)),
+                                            C.c_void_p(int(out)) if out else None,
+                                            C.c_void_p(int(scatter)), C.c_void_p(int(gather)),
+                                            _table(peers0), _table(peers1), sink_bytes, nelems, seq_no,
+                                            groups, subgroups, simd))
 
     def allgather_rank(self, algo, rank, inp, out, scatter, gather, peers0, peers1, sink_bytes, nelems,
                        seq_no, stream=None):

@@ -899,10 +899,10 @@ static int rank_sinks(const vr_ctx *ctx, int rank, void *scatter_buf, void *gath
 
 // One rank of an all-reduce, the form the reference constructs per process
 // (allreduce.hpp:18-28, parallel_transmit.hpp:36-60, bisect_transmit.hpp:427-482).
-extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
-                                 void *output, void *scatter_buf, void *gather_buf,
-                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
-                                 size_t nelems, uint32_t *seq_no) {
+static int allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
+                          void *scatter_buf, void *gather_buf, void *const peer_buf0[],
+                          void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no,
+                          uint32_t user_wires) {
   if (int rc = use_device(ctx)) return rc;
   const AlgoInfo *a = algo_info(algo);
   if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
@@ -938,12 +938,37 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
   if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
   const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};
   uint32_t seq = *seq_no, used = 0;
-  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, chunk_elems * 2, vec_halves, &seq, 0,
-                           &used, wlch))
+  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, chunk_elems * 2, vec_halves, &seq,
+                           user_wires, &used, wlch))
     return rc;
   *seq_no = seq + (used > geom.steps ? used : geom.steps);
   if (*seq_no == 0) *seq_no = 1;
   return VR_OK;
+}
+
+extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
+                                 void *output, void *scatter_buf, void *gather_buf,
+                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
+                                 size_t nelems, uint32_t *seq_no) {
+  return allreduce_rank(ctx, stream, algo, rank, input, output, scatter_buf, gather_buf, peer_buf0,
+                        peer_buf1, sink_bytes, nelems, seq_no, 0);
+}
+
+// testTransmit's per-rank form with a user grid (main.cpp:67-71, 289-294): every
+// rank launches groups x subgroups sub-groups of `simd` lanes.
+extern "C" int vr_allreduce_rank_grid(vr_ctx *ctx, void *stream, int algo, int rank, void *input,
+                                      void *output, void *scatter_buf, void *gather_buf,
+                                      void *const peer_buf0[], void *const peer_buf1[],
+                                      size_t sink_bytes, size_t nelems, uint32_t seq_no,
+                                      uint32_t groups, uint32_t subgroups, uint32_t simd) {
+  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
+  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
+  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
+  const uint64_t wires = (uint64_t)groups * subgroups;
+  uint32_t seq = seq_no;
+  return allreduce_rank(ctx, stream, algo, rank, input, output, scatter_buf, gather_buf, peer_buf0,
+                        peer_buf1, sink_bytes, nelems, &seq,
+                        wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires);
 }
 
 // One rank of the ring all-gather (AllGather(input, output, nelems, rank, seqNo, scatterBuf,

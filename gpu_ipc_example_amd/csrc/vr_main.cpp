@@ -191,8 +191,13 @@ int run_as_rank(const Options &o, int algo, size_t nelems) {
   vrank::check(vr_event_create(&ev1));
   auto run = [&](uint32_t flag) {
     uint32_t step = flag;
-    vrank::check(vr_allreduce_rank(ranks.get(), stream, algo, rank, input, nullptr, peerbuf0[rank],
-                                   peerbuf1[rank], peerbuf0, peerbuf1, sink, nelems, &step));
+    if (o.grid_given)       // testTransmit with the -g / -w / -s grid (main.cpp:67-71, 289-294)
+      vrank::check(vr_allreduce_rank_grid(ranks.get(), stream, algo, rank, input, nullptr, peerbuf0[rank],
+                                          peerbuf1[rank], peerbuf0, peerbuf1, sink, nelems, flag,
+                                          (uint32_t)o.groups, (uint32_t)o.subgroups, o.simd));
+    else
+      vrank::check(vr_allreduce_rank(ranks.get(), stream, algo, rank, input, nullptr, peerbuf0[rank],
+                                     peerbuf1[rank], peerbuf0, peerbuf1, sink, nelems, &step));
   };
   int status = 0;
   run((uint32_t)o.flag);

@@ -6,11 +6,17 @@
 //   AllGather<T, NRanks, Proto, Transmit, SubGroupSize>        (allgather.hpp:8-70)
 //   testTransmit<T>(std::string algo, ...) / testAllgather     (allreduce.cpp:1118-1213)
 // keeps its shape: construct, then launch on a stream; the protocol is chosen by
-// the <Proto, Transmit> template arguments or by the -a string.  What changes is
-// the meaning of "rank": the NRanks peers are virtual ranks, separate device
-// allocations inside one GPU, so one object drives all of them and the peer
-// scratch tables of the reference's constructor collapse into a VirtualRanks
-// handle.  Errors come back as the reference's std::logic_error texts.
+// the <Proto, Transmit> template arguments or by the -a string.  Two forms:
+//  * all ranks at once: the NRanks peers are virtual ranks, separate device
+//    allocations inside one GPU, one object drives all of them and the peer
+//    scratch tables of the reference's constructor collapse into a VirtualRanks
+//    handle;
+//  * one rank per object, with the reference's own constructor, launch() and
+//    testTransmit() parameter lists (input, scatterBuf / ipcbuf0, gatherBuf /
+//    ipcbuf1, peerBuf0[], peerBuf1[], rank, ...; a stream where the reference has a
+//    sycl::queue): the caller owns the scratch (scratchBytes()), N such launches
+//    on N streams or in N processes form one collective.
+// Errors come back as the reference's std::logic_error texts.
 //
 // Header-only; needs nothing but the C ABI (no HIP headers).  A stream is passed
 // as void* (a hipStream_t).
@@ -168,6 +174,32 @@ class VirtualRanks {
   int transport_ = VR_TRANSPORT_DEFAULT;
 };
 
+namespace detail {
+// The library context behind the one-rank-per-object form: one per world size and
+// process, on rankDevice() (set it before the first such object is built).
+inline int &rankDevice() {
+  static int device = 0;
+  return device;
+}
+inline VirtualRanks &rank_context(int nranks) {
+  static VirtualRanks *made[VR_MAX_RANKS + 1] = {};
+  if (nranks < 0 || nranks > VR_MAX_RANKS) throw std::logic_error("Unsupported communication topology");
+  if (!made[nranks]) made[nranks] = new VirtualRanks(nranks, rankDevice());
+  return *made[nranks];
+}
+inline std::size_t sink_bytes(VirtualRanks &ranks) {
+  std::size_t n = 0;
+  check(vr_rank_scratch_bytes(ranks.get(), &n));
+  return n;
+}
+}  // namespace detail
+
+// Bytes of scratch one rank of a world of `nranks` owns in the one-rank form: a
+// scatter sink followed by a gather sink (the reference's ipcbuf0 of
+// 2 * interm_size with ipcbuf1 = ipcbuf0 + interm_size, main.cpp:241-243).
+// Zero it once before the first launch (main.cpp:251).
+inline std::size_t scratchBytes(int nranks) { return 2 * detail::sink_bytes(detail::rank_context(nranks)); }
+
 struct LaunchParam {      // the nd_range getLaunchParam returns, in sub-group units
   std::uint32_t groups, subgroups, simd;
 };
@@ -194,6 +226,22 @@ struct AllReduce {
                              &workSize_));
   }
 
+  // The reference's own constructor (allreduce.hpp:18-28): this object is rank
+  // `rank` alone; scatterBuf / gatherBuf are its sinks, peerBuf0[] / peerBuf1[] every
+  // rank's (each of scratchBytes(NRanks) / 2 bytes).
+  AllReduce(T *input, std::size_t nelems, int rank, std::uint32_t seqNo, T *scatterBuf, T *gatherBuf,
+            T *const peerBuf0[], T *const peerBuf1[])
+      : ranks_(detail::rank_context(NRanks)), nelems_(nelems), seqNo_(seqNo), rank_(rank),
+        scatter_(scatterBuf), gather_(gatherBuf) {
+    for (int r = 0; r < NRanks; ++r) {
+      bufs_[r] = input;             // calcWorkSize sees this rank's pointer only
+      peer0_[r] = peerBuf0[r];
+      peer1_[r] = peerBuf1[r];
+    }
+    check(vr_check_allreduce(algo, NRanks, reinterpret_cast<const void *const *>(bufs_), nelems,
+                             &workSize_));
+  }
+
   LaunchParam getLaunchParam(std::uint32_t &updateSeqNo) const {
     vr_geometry g;
     check(vr_launch_geometry(algo, NRanks, nelems_, &g));
@@ -204,6 +252,11 @@ struct AllReduce {
   // Enqueue on `stream`; in place on the constructor's buffers.
   void operator()(void *stream = nullptr) {
     ranks_.setDtype(dtype_of<T>::value);
+    if (rank_ >= 0) {
+      check(vr_allreduce_rank(ranks_.get(), stream, algo, rank_, bufs_[0], nullptr, scatter_, gather_,
+                              peer0_, peer1_, detail::sink_bytes(ranks_), nelems_, &seqNo_));
+      return;
+    }
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
@@ -231,6 +284,17 @@ struct AllReduce {
     step = offload.seqNo_;
   }
 
+  // allreduce.hpp:64-74 with its own parameter list (a stream for the queue): one
+  // rank's launch; `step` advances like getLaunchParam does.
+  static void launch(T *input, T *ipcbuf0, T *ipcbuf1, T *const peerbuf0[], T *const peerbuf1[],
+                     std::size_t nelems, int rank, std::uint32_t &step, void *stream = nullptr) {
+    AllReduce offload(input, nelems, rank, step, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+  // Waits for `stream` and reports a poll time-out of one-rank launches.
+  static void wait(void *stream = nullptr) { detail::rank_context(NRanks).wait(stream); }
+
   std::size_t workSize() const { return workSize_; }
   std::uint32_t seqNo() const { return seqNo_; }
 
@@ -240,6 +304,9 @@ struct AllReduce {
   std::size_t nelems_;
   std::size_t workSize_ = 0;
   std::uint32_t seqNo_;
+  int rank_ = -1;                      // >= 0: one rank per object
+  void *scatter_ = nullptr, *gather_ = nullptr;
+  void *peer0_[VR_MAX_RANKS] = {}, *peer1_[VR_MAX_RANKS] = {};
 };
 
 // ---- bisectPAllReduce ---------------------------------------------------------------------
@@ -258,6 +325,19 @@ struct bisectPAllReduce {
     check(vr_check_allreduce(algo, NRanks, reinterpret_cast<const void *const *>(bufs_), nelems,
                              &workSize_));
   }
+  // The reference's own constructor (allreduce.hpp:220-232): one rank per object.
+  bisectPAllReduce(T *input, std::size_t nelems, int rank, std::uint32_t seqNo, T *scatterBuf,
+                   T *gatherBuf, T *const peerBuf0[], T *const peerBuf1[])
+      : ranks_(detail::rank_context(NRanks)), nelems_(nelems), seqNo_(seqNo), rank_(rank),
+        scatter_(scatterBuf), gather_(gatherBuf) {
+    for (int r = 0; r < NRanks; ++r) {
+      bufs_[r] = input;
+      peer0_[r] = peerBuf0[r];
+      peer1_[r] = peerBuf1[r];
+    }
+    check(vr_check_allreduce(algo, NRanks, reinterpret_cast<const void *const *>(bufs_), nelems,
+                             &workSize_));
+  }
   LaunchParam getLaunchParam(std::uint32_t &updateSeqNo) const {
     vr_geometry g;
     check(vr_launch_geometry(algo, NRanks, nelems_, &g));
@@ -266,6 +346,11 @@ struct bisectPAllReduce {
   }
   void operator()(void *stream = nullptr) {
     ranks_.setDtype(dtype_of<T>::value);
+    if (rank_ >= 0) {
+      check(vr_allreduce_rank(ranks_.get(), stream, algo, rank_, bufs_[0], nullptr, scatter_, gather_,
+                              peer0_, peer1_, detail::sink_bytes(ranks_), nelems_, &seqNo_));
+      return;
+    }
     check(vr_allreduce(ranks_.get(), stream, algo, ranks_.transportFor(algo), bufs_, nullptr, nelems_,
                        &seqNo_));
   }
@@ -281,6 +366,14 @@ struct bisectPAllReduce {
     offload(stream);
     step = offload.seqNo_;
   }
+  // allreduce.hpp:260-270 with its own parameter list.
+  static void launch(T *input, T *ipcbuf0, T *ipcbuf1, T *const peerbuf0[], T *const peerbuf1[],
+                     std::size_t nelems, int rank, std::uint32_t &step, void *stream = nullptr) {
+    bisectPAllReduce offload(input, nelems, rank, step, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+  static void wait(void *stream = nullptr) { detail::rank_context(NRanks).wait(stream); }
   std::size_t workSize() const { return workSize_; }
 
  private:
@@ -289,6 +382,9 @@ struct bisectPAllReduce {
   std::size_t nelems_;
   std::size_t workSize_ = 0;
   std::uint32_t seqNo_;
+  int rank_ = -1;
+  void *scatter_ = nullptr, *gather_ = nullptr;
+  void *peer0_[VR_MAX_RANKS] = {}, *peer1_[VR_MAX_RANKS] = {};
 };
 
 // ---- AllGather ----------------------------------------------------------------------------
@@ -314,9 +410,37 @@ struct AllGather {
     }
     check(vr_check_allgather(algo, NRanks, ins_, outs_, nelems, &workSize_));
   }
+  // The reference's own constructor (allgather.hpp:19-29): one rank per object.
+  AllGather(T *input, T *output, std::size_t nelems, int rank, std::uint32_t seqNo, T *scatterBuf,
+            T *gatherBuf, T *const peerBuf0[], T *const peerBuf1[])
+      : ranks_(detail::rank_context(NRanks)), nelems_(nelems), seqNo_(seqNo), rank_(rank),
+        scatter_(scatterBuf), gather_(gatherBuf) {
+    for (int r = 0; r < NRanks; ++r) {
+      ins_[r] = input;
+      outs_[r] = output;
+      peer0_[r] = peerBuf0[r];
+      peer1_[r] = peerBuf1[r];
+    }
+    check(vr_check_allgather(algo, NRanks, ins_, outs_, nelems, &workSize_));
+  }
   void operator()(void *stream = nullptr) {
+    ranks_.setDtype(dtype_of<T>::value);
+    if (rank_ >= 0) {
+      check(vr_allgather_rank(ranks_.get(), stream, algo, rank_, ins_[0], outs_[0], scatter_, gather_,
+                              peer0_, peer1_, detail::sink_bytes(ranks_), nelems_, &seqNo_));
+      return;
+    }
     check(vr_allgather(ranks_.get(), stream, algo, ranks_.transportFor(algo), ins_, outs_, nelems_, &seqNo_));
   }
+  // allgather.hpp:58-70 with its own parameter list.
+  static void launch(T *input, T *output, T *ipcbuf0, T *ipcbuf1, T *const peerbuf0[],
+                     T *const peerbuf1[], std::size_t nelems, int rank, std::uint32_t &step,
+                     void *stream = nullptr) {
+    AllGather offload(input, output, nelems, rank, step, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1);
+    offload(stream);
+    step = offload.seqNo_;
+  }
+  static void wait(void *stream = nullptr) { detail::rank_context(NRanks).wait(stream); }
   static void launch(VirtualRanks &ranks, T *const inputs[], T *const outputs[], std::size_t nelems,
                      std::uint32_t &step, void *stream = nullptr) {
     AllGather offload(ranks, inputs, outputs, nelems, step);
@@ -331,6 +455,9 @@ struct AllGather {
   std::size_t nelems_;
   std::size_t workSize_ = 0;
   std::uint32_t seqNo_;
+  int rank_ = -1;
+  void *scatter_ = nullptr, *gather_ = nullptr;
+  void *peer0_[VR_MAX_RANKS] = {}, *peer1_[VR_MAX_RANKS] = {};
 };
 
 // ---- string dispatch (the test-harness flavour) --------------------------------------------
@@ -360,6 +487,47 @@ void testAllgather(const std::string &transmitType, VirtualRanks &ranks, T *cons
   check(vr_allgather(ranks.get(), stream, algo, ranks.transportFor(algo),
                      reinterpret_cast<const void *const *>(const_cast<T **>(inputs)),
                      reinterpret_cast<void *const *>(const_cast<T **>(outputs)), nelems, &step));
+}
+
+// The reference's own test-harness entry (allreduce.hpp:337-343, main.cpp:67-71): one
+// rank's launch with a user grid, protocol by string; `queue` becomes a stream.
+template <typename T>
+void testTransmit(const std::string &transmitType, LaunchParam launchParam, T *input, T *ipcbuf0,
+                  T *ipcbuf1, T *const peerbuf0[], T *const peerbuf1[], std::size_t nelems, int rank,
+                  int world, std::uint32_t step, std::uint32_t subgroup, void *stream = nullptr) {
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
+  int algo = -1;
+  check(vr_algo_from_string(transmitType.c_str(), &algo));
+  if (vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
+  VirtualRanks &ranks = detail::rank_context(world);
+  ranks.setDtype(dtype_of<T>::value);
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  for (int r = 0; r < world; ++r) {
+    p0[r] = peerbuf0[r];
+    p1[r] = peerbuf1[r];
+  }
+  check(vr_allreduce_rank_grid(ranks.get(), stream, algo, rank, input, nullptr, ipcbuf0, ipcbuf1, p0, p1,
+                               detail::sink_bytes(ranks), nelems, step, launchParam.groups,
+                               launchParam.subgroups, subgroup));
+}
+
+// allreduce.hpp:345-348 / allreduce.cpp:1191-1213.
+template <typename T>
+void testAllgather(const std::string &transmitType, T *input, T *output, T *ipcbuf0, T *ipcbuf1,
+                   T *const peerbuf0[], T *const peerbuf1[], std::size_t nelems, int rank, int world,
+                   std::uint32_t &step, void *stream = nullptr) {
+  static_assert(sizeof(T) == 2, "this build moves 2-byte elements (binary16, bfloat16) only");
+  int algo = -1;
+  check(vr_algo_from_string(transmitType.c_str(), &algo));
+  if (!vr_algo_is_allgather(algo)) throw std::logic_error("Transmit type not support");
+  VirtualRanks &ranks = detail::rank_context(world);
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  for (int r = 0; r < world; ++r) {
+    p0[r] = peerbuf0[r];
+    p1[r] = peerbuf1[r];
+  }
+  check(vr_allgather_rank(ranks.get(), stream, algo, rank, input, output, ipcbuf0, ipcbuf1, p0, p1,
+                          detail::sink_bytes(ranks), nelems, &step));
 }
 
 }  // namespace vrank

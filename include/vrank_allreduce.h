@@ -188,6 +188,14 @@ int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void 
 int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
                       void *scatter_buf, void *gather_buf, void *const peer_buf0[],
                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+/* The same with the test harness's user grid (testTransmit<T>(algo, nd_range, input,
+ * ipcbuf0, ipcbuf1, peerbuf0, peerbuf1, nelems, rank, world, step, simd, queue),
+ * allreduce.hpp:337-343, main.cpp:67-71): `groups` x `subgroups` sub-groups per
+ * rank; every rank must pass the same grid.  Rejections as vr_allreduce_grid. */
+int vr_allreduce_rank_grid(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
+                           void *scatter_buf, void *gather_buf, void *const peer_buf0[],
+                           void *const peer_buf1[], size_t sink_bytes, size_t nelems,
+                           uint32_t seq_no, uint32_t groups, uint32_t subgroups, uint32_t simd);
 /* One rank of the ring all-gather, same contract (AllGather(input, output, nelems,
  * rank, seqNo, scatterBuf, gatherBuf, peerBuf0, peerBuf1), allgather.hpp:19-29):
  * output holds nranks * nelems elements; output + rank * nelems may be input. */

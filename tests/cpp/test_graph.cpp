@@ -128,6 +128,39 @@ int main() {
     VRCK(vr_ctx_check(ctx, stream));
   }
 
+  // The allocation-free wire all-reduce clears its sinks in every call and starts
+  // its flags from 1, so a captured call replays correctly: six replays with
+  // eager work in between, each compared with the oracle.
+  {
+    int parallel_id = -1;
+    VRCK(vr_algo_from_string("parallel", &parallel_id));
+    const std::vector<uint16_t> &sum = s1;       // the rotated-order sum of the inputs
+    hipGraph_t g3;
+    hipGraphExec_t e3;
+    HIPCK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    VRCK(vr_allreduce_static(ctx, stream, parallel_id, in, mid, n));
+    HIPCK(hipStreamEndCapture(stream, &g3));
+    HIPCK(hipGraphInstantiate(&e3, g3, nullptr, nullptr, 0));
+    for (int replay = 0; replay < 6; ++replay) {
+      for (int r = 0; r < N; ++r) HIPCK(hipMemsetAsync(mid[r], 0x3c, n * 2, stream));
+      // an eager call between replays leaves other flags in the shared sinks
+      if (replay % 2) VRCK(vr_allreduce_static(ctx, stream, bisect_id, in, out, n));
+      HIPCK(hipStreamSynchronize(stream));
+      HIPCK(hipGraphLaunch(e3, stream));
+      VRCK(vr_ctx_check(ctx, stream));
+      for (int r = 0; r < N; ++r) {
+        HIPCK(hipMemcpy(got.data(), mid[r], n * 2, hipMemcpyDeviceToHost));
+        const size_t bad = vro_count_mismatch(got.data(), sum.data(), n);
+        if (bad) {
+          printf("static replay %d rank %d: %zu mismatches\n", replay, r, bad);
+          ++failures;
+        }
+      }
+    }
+    (void)hipGraphExecDestroy(e3);
+    (void)hipGraphDestroy(g3);
+  }
+
   (void)hipGraphExecDestroy(exec);
   (void)hipGraphDestroy(graph);
   for (int r = 0; r < N; ++r) {

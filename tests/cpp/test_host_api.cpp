@@ -173,6 +173,97 @@ static int run_all() {
     }
     ranks.setDtype(VR_DTYPE_F16);
   }
+  // --- one rank per object: the reference's own constructor / launch / testTransmit lists -------------
+  // (allreduce.hpp:18-28, 64-74, 337-343; allgather.hpp:19-29): N launches on N streams of
+  // this process against scratch the caller owns (main.cpp:241-269).
+  {
+    const int W = 4;
+    void *streams[W] = {nullptr, nullptr, nullptr, nullptr};
+    for (int r = 1; r < W; ++r) check(vr_stream_create(0, &streams[r]));
+    const size_t sink = scratchBytes(W) / 2;
+    half_bits *ipcbuf0[W], *ipcbuf1[W];            // peerbuf0[i], peerbuf1[i] of main.cpp:260-269
+    for (int r = 0; r < W; ++r) {
+      void *p;
+      check(vr_malloc(0, 2 * sink, &p));
+      ipcbuf0[r] = (half_bits *)p;
+      ipcbuf1[r] = (half_bits *)((char *)p + sink);
+    }
+    auto zero = [&] { for (int r = 0; r < W; ++r) check(vr_memset(ipcbuf0[r], 0, 2 * sink)); };
+    auto wait_all = [&] { for (int r = 0; r < W; ++r) AllReduce<half_bits, W, Rt64_128, ParallelTransmit>::wait(streams[r]); };
+    uint32_t step = 0xe00f100f;
+    {  // AllReduce<...>::launch per rank
+      zero();
+      Ranks b(W, W * 4 * 5001, 81);
+      std::vector<uint16_t> want(b.nelems);
+      auto hp = b.host_ptrs();
+      vro_allreduce_rotated(want.data(), hp.data(), W, b.nelems);
+      uint32_t next = step;
+      for (int r = 0; r < W; ++r) {
+        next = step;
+        AllReduce<half_bits, W, Rt64_128, ParallelTransmit>::launch(b.dev[r], ipcbuf0[r], ipcbuf1[r], ipcbuf0,
+                                                                    ipcbuf1, b.nelems, r, next, streams[r]);
+      }
+      wait_all();
+      EXPECT(next > step);
+      step = next;
+      EXPECT(b.mismatches(want) == 0);
+    }
+    {  // bisectPAllReduce constructed per rank, then called
+      zero();
+      Ranks b(W, W * 4 * 3333, 82);
+      std::vector<uint16_t> want(b.nelems);
+      auto hp = b.host_ptrs();
+      vro_allreduce_bisect(want.data(), hp.data(), W, b.nelems);
+      for (int r = 0; r < W; ++r) {
+        bisectPAllReduce<half_bits, W> ar(b.dev[r], b.nelems, r, step, ipcbuf0[r], ipcbuf1[r], ipcbuf0, ipcbuf1);
+        EXPECT(ar.workSize() == b.nelems * 2 / W);
+        ar(streams[r]);
+      }
+      wait_all();
+      step += 1000;
+      EXPECT(b.mismatches(want) == 0);
+    }
+    {  // testTransmit<T>(algo, nd_range, input, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1, nelems, rank, world, step, simd, queue)
+      for (const char *algo : {"small", "simple_ring"}) {
+        zero();
+        Ranks b(W, 14336, 83);
+        std::vector<uint16_t> want(b.nelems);
+        auto hp = b.host_ptrs();
+        vro_allreduce_rotated(want.data(), hp.data(), W, b.nelems);
+        for (int r = 0; r < W; ++r)
+          testTransmit<half_bits>(algo, {7, 8, 16}, b.dev[r], ipcbuf0[r], ipcbuf1[r], ipcbuf0, ipcbuf1, b.nelems,
+                                  r, W, step, 16, streams[r]);
+        wait_all();
+        step += 1000;
+        EXPECT(b.mismatches(want) == 0);
+      }
+    }
+    {  // AllGather per rank
+      zero();
+      Ranks in(W, 8 * 999, 84), out(W, 8 * 999, 85, W);
+      std::vector<uint16_t> want(W * in.nelems);
+      auto hp = in.host_ptrs();
+      vro_allgather(want.data(), hp.data(), W, in.nelems);
+      for (int r = 0; r < W; ++r) {
+        uint32_t s2 = step;
+        AllGather<half_bits, W, Rt64_128_PCIE, RingTransmit>::launch(in.dev[r], out.dev[r], ipcbuf0[r], ipcbuf1[r],
+                                                                     ipcbuf0, ipcbuf1, in.nelems, r, s2, streams[r]);
+      }
+      wait_all();
+      EXPECT(out.mismatches(want) == 0);
+    }
+    {  // the constructor's exceptions, per rank
+      Ranks b(W, W * 64, 86);
+      EXPECT(thrown([&] { AllReduce<half_bits, W, Rt64, ParallelTransmit> a((half_bits *)((char *)b.dev[0] + 4), b.nelems, 0, 1, ipcbuf0[0], ipcbuf1[0], ipcbuf0, ipcbuf1); }) ==
+             "We only support aligned pointer for now");
+      EXPECT(thrown([&] { AllReduce<half_bits, W, Rt64, ParallelTransmit> a(b.dev[0], W * 4 + 4, 0, 1, ipcbuf0[0], ipcbuf1[0], ipcbuf0, ipcbuf1); }) ==
+             "We don't support non-even divide yet");
+      EXPECT(thrown([&] { testTransmit<half_bits>("tree", {1, 4, 16}, b.dev[0], ipcbuf0[0], ipcbuf1[0], ipcbuf0, ipcbuf1, b.nelems, 0, W, 1, 16); }) ==
+             "Transmit type not support");
+    }
+    for (int r = 0; r < W; ++r) vr_free(ipcbuf0[r]);
+    for (int r = 1; r < W; ++r) vr_stream_destroy(streams[r]);
+  }
   // --- the reference's exceptions -------------------------------------------------------------------------
   {
     VirtualRanks ranks(8), two(2);
