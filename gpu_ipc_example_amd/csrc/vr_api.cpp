@@ -470,7 +470,8 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   // Inputs and outputs that cannot stay in the 256 MiB memory-side cache anyway are
   // streamed past it, which leaves that cache to the sinks (measured: faster from
   // 256 MiB of inputs + outputs on, slower below).
-  const size_t io_bytes = 2 * (size_t)N * chunk_bytes * (a->allgather ? 1 : (size_t)N);
+  const size_t io_bytes = a->allgather ? (size_t)N * chunk_bytes * (1 + (size_t)N)    // N slices in, N x N out
+                                       : 2 * (size_t)N * chunk_bytes * (size_t)N;     // N chunks per rank, in + out
   args.stream_io = c->tune.wire_stream_io >= 0 ? (uint32_t)c->tune.wire_stream_io
                                                : (io_bytes >= (256ull << 20) ? 1u : 0u);
   const bool solo = wlch.solo_rank >= 0;
