@@ -541,6 +541,7 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   uint32_t *status = nullptr;
   HIP_TRY(hipMalloc((void **)&status, 256));
   hipError_t e = hipMemset(status, 0, 256);
+  if (e == hipSuccess) e = hipStreamSynchronize(nullptr);   // the fill has run before any stream may read the word
   void *fixed = nullptr;
   size_t fixed_bytes = 0;
   if (e == hipSuccess) e = wire_static_scratch(device, &fixed, &fixed_bytes);
@@ -1089,6 +1090,7 @@ static int check_status_word(uint32_t *word, bool *timed_out) {
   HIP_TRY(hipMemcpy(&status, word, sizeof status, hipMemcpyDeviceToHost));
   if (status != 0) {
     HIP_TRY(hipMemset(word, 0, sizeof status));
+    HIP_TRY(hipStreamSynchronize(nullptr));
     *timed_out = true;
   }
   return VR_OK;
@@ -1399,6 +1401,9 @@ extern "C" int vr_free(void *ptr) {
 
 extern "C" int vr_memset(void *ptr, int value, size_t bytes) {
   HIP_TRY(hipMemset(ptr, value, bytes));
+  // hipMemset of device memory may return before the fill has run; callers zero
+  // scratch that kernels on other streams, or other processes, write into next.
+  HIP_TRY(hipStreamSynchronize(nullptr));
   return VR_OK;
 }
 

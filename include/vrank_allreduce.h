@@ -337,7 +337,7 @@ int vr_device_count(int *count);
 int vr_device_name(int device, char *buf, size_t buflen);
 int vr_malloc(int device, size_t bytes, void **out);
 int vr_free(void *ptr);
-int vr_memset(void *ptr, int value, size_t bytes);
+int vr_memset(void *ptr, int value, size_t bytes);                 /* complete on return */
 int vr_copy_to_device(void *dst, const void *src_host, size_t bytes);
 int vr_copy_to_host(void *dst_host, const void *src, size_t bytes);
 int vr_stream_create(int device, void **stream_out);
