@@ -38,7 +38,8 @@ def run_ranks(world, extra, per_rank=None, timeout=100):
 
 
 @pytest.mark.parametrize("world,algo", [(2, "simple"), (4, "simple"), (2, "small"), (4, "bisect"),
-                                        (4, "parallel"), (2, "simple_ring"), (4, "small_pcie")])
+                                        (4, "parallel"), (2, "simple_ring"), (4, "small_pcie"),
+                                        (8, "simple"), (8, "bisect")])
 def test_fill_pattern_verify_across_processes(world, algo):
     """main.cpp's -v flow in every rank process: fill_pattern inputs, the host sum
     of allreduce.cpp:18-27 as the check."""
@@ -50,7 +51,7 @@ def test_fill_pattern_verify_across_processes(world, algo):
 
 
 @pytest.mark.parametrize("world,algo", [(2, "parallel"), (4, "parallel"), (4, "bisect"), (4, "simple_ring"),
-                                        (2, "small")])
+                                        (2, "small"), (8, "parallel"), (8, "bisect")])
 def test_seeded_inputs_match_the_oracle_across_processes(oracle, tmp_path, world, algo):
     n = 1 << 20
     seed = 9100 + world
@@ -70,6 +71,18 @@ def test_timed_run_protocol_across_processes():
     res = run_ranks(4, ["-n", "1M", "-a", "simple"])
     for r, (rc, text) in enumerate(res):
         assert rc == 0 and "[%d] Running time: " % r in text, (r, text)
+
+
+def test_headline_shape_as_eight_processes():
+    """8 rank processes, bisect, 32 MiB per rank: the reference's `mpirun -np 8 ./main
+    -a bisect -n 16M` on one GPU, with the user grid of its test scripts."""
+    res = run_ranks(8, ["-n", "16M", "-a", "bisect"])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0 and "[%d] Running time: " % r in text, (r, text)
+    print("\n".join(text.strip().splitlines()[-1] for _, text in res))
+    res = run_ranks(8, ["-v", "-n", "14336", "-a", "small", "-g", "7", "-w", "8"])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0 and "match the host sum" in text, (r, text)
 
 
 def test_a_missing_rank_is_a_time_out_not_a_hang():
