@@ -22,12 +22,9 @@
 #include <string>
 #include <vector>
 
-#include "vr_internal.h"
+#include "vr_host.h"
 
-namespace vr {
-int api_fail(int status, const std::string &detail);   // vr_api.cpp: records the thread's error detail
-}
-using vr::api_fail;
+static int api_fail(int status, const std::string &detail) { return vr::fail(status, detail); }
 
 namespace {
 
