@@ -1,4 +1,4 @@
-// Internal interface between the C ABI (vr_api.cpp) and the gfx950 kernels.
+// Internal interface between the C ABI (vr_api.cpp, vr_wire_host.cpp) and the gfx950 kernels.
 #pragma once
 
 #include <hip/hip_runtime.h>

@@ -1,6 +1,6 @@
 // Sink geometry of the wire transport: which message slot of a rank's scatter or
 // gather sink a wave touches, for every flow.  The kernels (vr_wire.hip), the host
-// code that sizes the scratch (vr_api.cpp) and a CPU bounds test all use these
+// code that sizes the scratch (vr_wire_host.cpp) and a CPU bounds test all use these
 // same functions, so a sink can be proven large enough without a GPU.
 //
 // A sink is `slots` message slots of kSlotBytesMax bytes followed by `slots`
