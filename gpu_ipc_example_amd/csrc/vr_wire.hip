@@ -1098,6 +1098,8 @@ static void *g_static_ptr[kMaxDevices];
 
 hipError_t wire_static_scratch(int device, void **ptr, size_t *bytes) {
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  static std::mutex lock;   // contexts may be created from several threads
+  std::lock_guard<std::mutex> hold(lock);
   if (!g_static_ptr[device]) {
     // The caller has made `device` current: each GPU holds its own copy of the
     // array at its own address.
