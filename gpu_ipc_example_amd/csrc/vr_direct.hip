@@ -64,7 +64,9 @@ __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, uint32_t off, V v) 
 // `owner`, and the chunk index itself.
 template <int N, int ORDER>
 __device__ __forceinline__ int chunk_of_owner(int owner) {
-  if constexpr (ORDER == ORDER_BISECT)
+  // (The no-add yardstick stands beside the bisect all-reduce, so it deals the
+  // chunks to the work-groups, and thereby to the XCDs, the same way.)
+  if constexpr (ORDER == ORDER_BISECT || ORDER == ORDER_COPY)
     return (owner & 1) * (N / 2) + (owner >> 1);
   else
     return owner;
