@@ -72,6 +72,13 @@ def lib():
         "vr_allreduce_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
         "vr_allgather_rank": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, C.POINTER(u32)]),
         "vr_allreduce_rank_grid": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, u32, u32, u32, u32]),
+        "vr_allgather_rank_grid": (i, [vp, vp, i, i, vp, vp, vp, vp, vpp, vpp, sz, sz, u32, u32, u32, u32]),
+        "vr_allreduce_ranks": (i, [vp, vp, i, i, i, vpp, vpp, vpp, vpp, sz, sz, C.POINTER(u32)]),
+        "vr_allgather_ranks": (i, [vp, vp, i, i, i, vpp, vpp, vpp, vpp, sz, sz, C.POINTER(u32)]),
+        "vr_allgather_grid": (i, [vp, vp, i, i, vpp, vpp, sz, u32, u32, u32, u32]),
+        "vr_time_allreduce_grouped": (i, [vp, vp, i, i, vpp, vpp, sz, i, i, C.POINTER(C.c_float),
+                                          C.POINTER(C.c_double)]),
+        "vr_rank_flags_used": (i, [vp, i, sz, u32, u32, C.POINTER(u32)]),
         "vr_rank_scratch_bytes": (i, [vp, C.POINTER(sz)]),
         "vr_allreduce_static": (i, [vp, vp, i, vpp, vpp, sz]),
         "vr_ctx_set_dtype": (i, [vp, i]),
@@ -267,6 +274,11 @@ class VirtualRanks:
         _check(lib().vr_rank_scratch_bytes(self._h, C.byref(out)))
         return out.value
 
+    def rank_flags_used(self, algo, nelems, groups=0, subgroups=0):
+        out = C.c_uint32(0)
+        _check(lib().vr_rank_flags_used(self._h, algo_id(algo), nelems, groups, subgroups, C.byref(out)))
+        return out.value
+
     def allreduce_rank(self, algo, rank, inp, scatter, gather, peers0, peers1, sink_bytes, nelems,
                        seq_no, out=None, stream=None):
         """One rank's wires against caller-owned sinks; returns the advanced sequence number."""
@@ -294,6 +306,30 @@ class VirtualRanks:
                                        C.c_void_p(int(out)), C.c_void_p(int(scatter)),
                                        C.c_void_p(int(gather)), _table(peers0), _table(peers1),
                                        sink_bytes, nelems, C.byref(seq)))
+        return seq.value
+
+    def allgather_rank_grid(self, algo, rank, inp, out, scatter, gather, peers0, peers1, sink_bytes, nelems,
+                            seq_no, groups, subgroups, simd=16, stream=None):
+        _check(lib().vr_allgather_rank_grid(self._h, stream, algo_id(algo), rank, C.c_void_p(int(inp)),
+                                            C.c_void_p(int(out)), C.c_void_p(int(scatter)),
+                                            C.c_void_p(int(gather)), _table(peers0), _table(peers1),
+                                            sink_bytes, nelems, seq_no, groups, subgroups, simd))
+
+    def allreduce_ranks(self, algo, first, inputs, peers0, peers1, sink_bytes, nelems, seq_no, outs=None,
+                        stream=None):
+        """Ranks [first, first + len(inputs)) in one launch; returns the advanced sequence number."""
+        seq = C.c_uint32(seq_no)
+        _check(lib().vr_allreduce_ranks(self._h, stream, algo_id(algo), first, len(inputs), _table(inputs),
+                                        _table(outs) if outs is not None else None, _table(peers0),
+                                        _table(peers1), sink_bytes, nelems, C.byref(seq)))
+        return seq.value
+
+    def allgather_ranks(self, algo, first, inputs, outputs, peers0, peers1, sink_bytes, nelems, seq_no,
+                        stream=None):
+        seq = C.c_uint32(seq_no)
+        _check(lib().vr_allgather_ranks(self._h, stream, algo_id(algo), first, len(inputs), _table(inputs),
+                                        _table(outputs), _table(peers0), _table(peers1), sink_bytes,
+                                        nelems, C.byref(seq)))
         return seq.value
 
     def allreduce_static(self, algo, bufs, nelems, outs=None, stream=None):
@@ -332,6 +368,12 @@ class VirtualRanks:
         _check(lib().vr_allgather(self._h, stream, algo_id(algo), transport, _table(inputs),
                                   _table(outputs), nelems, C.byref(self.seq_no)))
 
+    def allgather_grid(self, algo, inputs, outputs, nelems, groups, subgroups, simd=16,
+                       transport=TRANSPORT_DEFAULT, stream=None, seq_no=0xE00F100F):
+        self._reserve_for(algo, transport)
+        _check(lib().vr_allgather_grid(self._h, stream, algo_id(algo), transport, _table(inputs),
+                                       _table(outputs), nelems, seq_no, groups, subgroups, simd))
+
     def check(self, stream=None):
         _check(lib().vr_ctx_check(self._h, stream))
 
@@ -345,6 +387,18 @@ class VirtualRanks:
         _check(lib().vr_time_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
                                        _table(outs) if outs is not None else None, nelems, iters, ms))
         return np.frombuffer(ms, np.float32).copy()
+
+    def time_allreduce_grouped(self, algo, bufs, nelems, groups, per_group, outs=None,
+                               transport=TRANSPORT_DEFAULT, stream=None):
+        """(ms per launch for each group, host microseconds one vr_allreduce call takes), both
+        measured inside the library around calls made like any caller's."""
+        ms = (C.c_float * groups)()
+        host_us = C.c_double(0.0)
+        self._reserve_for(algo, transport)
+        _check(lib().vr_time_allreduce_grouped(self._h, stream, algo_id(algo), transport, _table(bufs),
+                                               _table(outs) if outs is not None else None, nelems,
+                                               groups, per_group, ms, C.byref(host_us)))
+        return np.frombuffer(ms, np.float32).copy(), host_us.value
 
     def time_allgather(self, algo, inputs, outputs, nelems, iters, transport=TRANSPORT_DEFAULT,
                        stream=None):

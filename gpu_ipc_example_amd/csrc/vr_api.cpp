@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include <string>
 #include <vector>
@@ -283,8 +284,10 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
          !strcmp(key, "wire_cooperative")) &&
         !(value == 0 || value == 1))
       return fail(VR_ERR_INVALID, "flag must be 0, 1 or -1 (automatic)");
-    if (!strcmp(key, "wire_fenced") && (value < 0 || value > 2))
-      return fail(VR_ERR_INVALID, "wire_fenced must be 0 (embedded flags), 1 (flag words with fences), 2 (8-byte messages) or -1");
+    if (!strcmp(key, "wire_fenced") && (value < 0 || value > 4))
+      return fail(VR_ERR_INVALID, "wire_fenced must be 0 (embedded flags), 1 (flag words with fences), 2 (8-byte messages), "
+                                  "3 (flag words with fences, payload written through), 4 (flag words, agent-scope "
+                                  "accesses ordered by store completion) or -1");
     if (!strcmp(key, "nt_store") && (value < 0 || value > 2))
       return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
     if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))
@@ -474,34 +477,45 @@ extern "C" int vr_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, 
   return VR_OK;
 }
 
+// The test harness's grid (main.cpp:289-294): rejections in the reference's order
+// (main.cpp:289-291, then allreduce.cpp:852/917), then its mapping onto this
+// device.  Direct transport: a block holds the same number of lanes (rounded to
+// whole waves, at most 1024) and the launch holds ceil(groups / nranks) blocks for
+// every virtual rank.  Wire transport: groups x subgroups is the number of
+// sub-groups (wires) per rank.
+static int apply_user_grid(const vr_ctx *ctx, uint32_t groups, uint32_t subgroups, uint32_t simd,
+                           Tuning *t, uint32_t *wires) {
+  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
+  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
+  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
+  size_t lanes = (size_t)subgroups * simd;
+  lanes = ((lanes + 63) / 64) * 64;
+  if (lanes > 1024) lanes = 1024;
+  t->block = (int)lanes;
+  t->unroll = 1;
+  t->oneshot = 0;
+  t->force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
+  const uint64_t w = (uint64_t)groups * subgroups;
+  *wires = w > 0xffffffffull ? 0xffffffffu : (uint32_t)w;
+  return VR_OK;
+}
+
 extern "C" int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transport,
                                  void *const bufs[], void *const outs[], size_t nelems,
                                  uint32_t seq_no, uint32_t groups, uint32_t subgroups,
                                  uint32_t simd) {
-  // main.cpp:289-291, then allreduce.cpp:852/917.
-  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
-  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
-  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  Tuning grid;
+  uint32_t wires = 0;
+  if (int rc = apply_user_grid(ctx, groups, subgroups, simd, &grid, &wires)) return rc;
   Prepared p;
   if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
   int tr;
   if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
-  // Map the reference's (groups x subgroups x simd) grid onto wavefronts: a block
-  // holds the same number of lanes (rounded to whole waves, at most 1024) and the
-  // launch holds ceil(groups / nranks) blocks for every virtual rank.
   Tuning t = tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place);
-  size_t lanes = (size_t)subgroups * simd;
-  lanes = ((lanes + 63) / 64) * 64;
-  if (lanes > 1024) lanes = 1024;
-  t.block = (int)lanes;
-  t.unroll = 1;
-  t.oneshot = 0;
-  t.force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
-  // Wire transport: groups x subgroups is the number of sub-groups (wires) per rank.
-  const uint64_t wires = (uint64_t)groups * subgroups;
+  (void)apply_user_grid(ctx, groups, subgroups, simd, &t, &wires);
   uint32_t next = 0;
-  return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no,
-                       wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, &next);
+  return run_allreduce(ctx, (hipStream_t)stream, p, tr, t, seq_no, wires, &next);
 }
 
 struct PreparedGather {
@@ -546,30 +560,59 @@ static int prepare_allgather(vr_ctx *ctx, int algo, const void *const inputs[],
   return vr_launch_geometry(algo, N, nelems, &p->geom);
 }
 
+// Runs one all-gather starting at sequence number `seq_no`; *next_seq receives
+// the sequence number the following launch should start at.
+static int run_allgather(vr_ctx *ctx, hipStream_t s, const PreparedGather &p, int transport,
+                         const Tuning &t, size_t nelems, uint32_t seq_no, uint32_t user_wires,
+                         uint32_t *next_seq) {
+  if (transport == VR_TRANSPORT_WIRE) {
+    uint32_t used = 0, start = seq_no;
+    if (int rc = wire_launch_ctx(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start, user_wires, &used))
+      return rc;
+    *next_seq = start + (used > p.geom.steps ? used : p.geom.steps);
+    if (*next_seq == 0) *next_seq = 1;
+    return VR_OK;
+  }
+  if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
+  hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);
+  if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
+  *next_seq = seq_no + p.geom.steps;
+  if (*next_seq == 0) *next_seq = 1;
+  return VR_OK;
+}
+
+static Tuning allgather_tuning(const vr_ctx *ctx, const AlgoInfo *a, size_t nelems) {
+  const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
+  return tuning_for(ctx, a, in_bytes, in_bytes * ctx->nranks, false);
+}
+
 extern "C" int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
                             const void *const inputs[], void *const outputs[], size_t nelems,
                             uint32_t *seq_no) {
   PreparedGather p;
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
   uint32_t *seq = seq_no ? seq_no : &ctx->seq_no;
-  if (transport == VR_TRANSPORT_WIRE) {
-    uint32_t used = 0, start = *seq;
-    if (int rc = wire_launch_ctx(ctx, (hipStream_t)stream, p.a, p.in, p.out, nelems * 2, p.vec_halves,
-                                 &start, 0, &used))
-      return rc;
-    *seq = start + (used > p.geom.steps ? used : p.geom.steps);
-    if (*seq == 0) *seq = 1;
-    return VR_OK;
-  }
-  if (transport != VR_TRANSPORT_DEFAULT && transport != VR_TRANSPORT_DIRECT) return fail(VR_ERR_INVALID, "bad transport");
-  const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
-  hipError_t e = launch_direct_allgather((hipStream_t)stream, ctx->dev,
-                                         tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false),
-                                         ctx->nranks, p.in, p.out, nelems, p.vec_halves);
-  if (e != hipSuccess) return fail_hip(e, "launch_direct_allgather");
-  *seq += p.geom.steps;
-  if (*seq == 0) *seq = 1;
+  uint32_t next = *seq;
+  if (int rc = run_allgather(ctx, (hipStream_t)stream, p, transport, allgather_tuning(ctx, p.a, nelems), nelems,
+                             *seq, 0, &next))
+    return rc;
+  *seq = next;
   return VR_OK;
+}
+
+extern "C" int vr_allgather_grid(vr_ctx *ctx, void *stream, int algo, int transport,
+                                 const void *const inputs[], void *const outputs[], size_t nelems,
+                                 uint32_t seq_no, uint32_t groups, uint32_t subgroups, uint32_t simd) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  Tuning grid;
+  uint32_t wires = 0;
+  if (int rc = apply_user_grid(ctx, groups, subgroups, simd, &grid, &wires)) return rc;
+  PreparedGather p;
+  if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
+  Tuning t = allgather_tuning(ctx, p.a, nelems);
+  (void)apply_user_grid(ctx, groups, subgroups, simd, &t, &wires);
+  uint32_t next = 0;
+  return run_allgather(ctx, (hipStream_t)stream, p, transport, t, nelems, seq_no, wires, &next);
 }
 
 // ---------------------------------------------------------------------------------
@@ -633,20 +676,62 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
                                  int iters, float *ms_out) {
   PreparedGather p;
   if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
-  const size_t in_bytes = (size_t)ctx->nranks * nelems * 2;
-  const Tuning t = tuning_for(ctx, p.a, in_bytes, in_bytes * ctx->nranks, false);
+  const Tuning t = allgather_tuning(ctx, p.a, nelems);
   hipStream_t s = (hipStream_t)stream;
   return time_launches(s, iters, ms_out, [&]() -> int {
-    if (transport == VR_TRANSPORT_WIRE) {
-      uint32_t used = 0, start = ctx->seq_no;
-      int rc = wire_launch_ctx(ctx, s, p.a, p.in, p.out, nelems * 2, p.vec_halves, &start, 0, &used);
-      ctx->seq_no = start + (used > p.geom.steps ? used : p.geom.steps);
-      if (ctx->seq_no == 0) ctx->seq_no = 1;
-      return rc;
-    }
-    hipError_t e = launch_direct_allgather(s, ctx->dev, t, ctx->nranks, p.in, p.out, nelems, p.vec_halves);
-    return e == hipSuccess ? VR_OK : fail_hip(e, "launch_direct_allgather");
+    uint32_t next = ctx->seq_no;
+    int rc = run_allgather(ctx, s, p, transport, t, nelems, ctx->seq_no, 0, &next);
+    ctx->seq_no = next;
+    return rc;
   });
+}
+
+// `groups` event pairs, each around `per_group` back-to-back vr_allreduce calls made
+// exactly as a caller makes them (validation, launch heuristics and launch in every
+// call).  ms_out[g] = device time of group g divided by per_group; *host_call_us
+// (optional) = host wall time one vr_allreduce call took to return, averaged over
+// all of them.
+extern "C" int vr_time_allreduce_grouped(vr_ctx *ctx, void *stream, int algo, int transport,
+                                         void *const bufs[], void *const outs[], size_t nelems,
+                                         int groups, int per_group, float *ms_out,
+                                         double *host_call_us) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (groups <= 0 || per_group <= 0 || !ms_out) return fail(VR_ERR_INVALID, "groups, per_group > 0 and ms_out");
+  if (groups > 4096) return fail(VR_ERR_INVALID, "at most 4096 groups");
+  if (int rc = use_device(ctx)) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  std::vector<hipEvent_t> ev(2 * (size_t)groups, nullptr);
+  int rc = VR_OK;
+  for (auto &e : ev)
+    if (hipError_t err = hipEventCreate(&e); err != hipSuccess) { rc = fail_hip(err, "hipEventCreate"); break; }
+  double host_s = 0.0;
+  for (int g = 0; g < groups && rc == VR_OK; ++g) {
+    if (hipEventRecord(ev[2 * g], s) != hipSuccess) rc = fail(VR_ERR_HIP, "hipEventRecord");
+    timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (int i = 0; i < per_group && rc == VR_OK; ++i)
+      rc = vr_allreduce(ctx, stream, algo, transport, bufs, outs, nelems, nullptr);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    host_s += (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+    if (rc == VR_OK && hipEventRecord(ev[2 * g + 1], s) != hipSuccess) rc = fail(VR_ERR_HIP, "hipEventRecord");
+    // keep the queue short: a group is waited for before the one after next is issued
+    if (rc == VR_OK && g >= 1)
+      if (hipError_t err = hipEventSynchronize(ev[2 * (g - 1) + 1]); err != hipSuccess) rc = fail_hip(err, "hipEventSynchronize");
+  }
+  if (rc == VR_OK)
+    if (hipError_t err = hipStreamSynchronize(s); err != hipSuccess) rc = fail_hip(err, "hipStreamSynchronize");
+  for (int g = 0; g < groups && rc == VR_OK; ++g) {
+    float ms = 0.f;
+    if (hipError_t err = hipEventElapsedTime(&ms, ev[2 * g], ev[2 * g + 1]); err != hipSuccess) {
+      rc = fail_hip(err, "hipEventElapsedTime");
+      break;
+    }
+    ms_out[g] = ms / (float)per_group;
+  }
+  for (auto &e : ev)
+    if (e) (void)hipEventDestroy(e);
+  if (rc == VR_OK && host_call_us) *host_call_us = host_s * 1e6 / ((double)groups * per_group);
+  return rc;
 }
 
 // The probes are pure streaming: streaming loads, streaming agent-scope stores,

@@ -107,7 +107,6 @@ struct vr_ctx {
   vr::DType dtype = vr::DT_F16;
   uint32_t *status = nullptr;     // time-out word of this context's wire launches (256 B)
   vr::WireState wire;
-  bool static_used = false;       // vr_allreduce_static has run on this context
 };
 
 namespace vr {

@@ -75,11 +75,16 @@ enum WireFormat : int {
   WIRE_FMT_FLAG = 2,  // 16 B payload lines + one fenced flag word per message
   WIRE_FMT_LL16 = 3,  // 8 B payload + the flag twice per 16-byte store (Rt64_PCIE family)
   WIRE_FMT_RT256 = 4, // the reference's 256-byte message: 240 B payload, a flag per 64 bytes (Rt64_128_PCIE)
+  WIRE_FMT_FLAG_WT = 5,      // WIRE_FMT_FLAG with the payload stored written through at agent scope
+  WIRE_FMT_FLAG_SCOPED = 6,  // flag words, every access at agent scope, ordered by store completion: no fences
 };
+static inline bool wire_fmt_is_flag(int fmt) {
+  return fmt == WIRE_FMT_FLAG || fmt == WIRE_FMT_FLAG_WT || fmt == WIRE_FMT_FLAG_SCOPED;
+}
 constexpr int kWireMaxSlots = 8;     // deepest slot ring any flow uses
 
 struct WireArgs {
-  PtrTable in, out;          // per-rank input / output (a one-rank launch fills only its own entry)
+  PtrTable in, out;          // per-rank input / output (only the entries of the ranks the launch holds)
   PtrTable scatter, gather;  // per-rank sinks (the reference's peerBuf0[] / peerBuf1[])
   size_t flag_off;           // byte offset of the flag words inside a sink (WIRE_FMT_FLAG)
   size_t chunk_bytes;        // bytes per rank-chunk (all-gather: bytes of one slice)
@@ -87,7 +92,8 @@ struct WireArgs {
   uint32_t seq;              // first flag value of this launch
   uint32_t spin_limit;
   uint32_t ahead;            // steps the scatters of the parallel flow run ahead of its gathers
-  int solo_rank;             // >= 0: the grid holds this one rank's wires only; -1: block b is rank b % N
+  int rank_first, rank_count; // the grid holds the wires of ranks [rank_first, rank_first + rank_count):
+                             // block b is rank rank_first + b % rank_count (all ranks: 0, N)
   uint32_t stream_io;        // 1: inputs are loaded and outputs stored with streaming cache policies
   uint32_t *status;          // non-zero once any poll gave up
 };
@@ -101,6 +107,12 @@ hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_hal
                        uint32_t blocks, uint32_t block_threads, WireArgs &args, bool cooperative,
                        DType dtype);
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes);
+// Bytes of a message slot in the sinks for a format.
+uint32_t wire_slot_bytes(WireFormat fmt, int vec_halves);
+// Clears, in every rank's scatter and gather sink, the first `slot_bytes` bytes
+// and `flag_bytes` bytes of flag words at `flag_off`.
+hipError_t launch_wire_clear_sinks(hipStream_t s, const PtrTable &scatter, const PtrTable &gather, int nranks,
+                                   size_t slot_bytes, size_t flag_off, size_t flag_bytes);
 // The library's own fixed scratch region in device memory (one per GPU, held
 // until the process ends): its device address on the current device and its size.
 constexpr uint32_t kStaticWiresPerRank = 32;

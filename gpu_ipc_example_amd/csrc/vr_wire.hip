@@ -1,9 +1,9 @@
 // Wire transport: the reference's message-passing stage structure on one GPU.
 //
 // One persistent kernel holds the work-groups of ALL virtual ranks (block b
-// belongs to rank b % N), or, launched once per rank (WireArgs::solo_rank), the
-// work-groups of one rank only, as one process per GPU would run it.  A
-// wavefront plays the part of
+// belongs to rank b % N), or of a group of consecutive ranks (WireArgs::rank_first,
+// rank_count): one rank per launch is how one process per GPU would run it, k
+// ranks per launch is k ranks per process.  A wavefront plays the part of
 // a reference sub-group ("wire"): it loads its rank's input, pushes messages
 // into peers' scatter/gather sinks in device scratch, polls its own sinks, adds
 // in the reference's order and stores.  Sink indexing, slot rotation and flag
@@ -156,6 +156,7 @@ template <int U, int DT>
 struct WireLL {
   static constexpr uint32_t kWireBytes = 64u * 4u * U;   // payload one wave moves per step
   static constexpr uint32_t kSlotBytes = 64u * 8u * U;   // message bytes in the sink
+  static constexpr bool kBatchSends = false;   // the flag travels inside every message
   struct Reg {
     uint32_t d[U];
   };
@@ -189,6 +190,20 @@ struct WireLL {
       __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, msg, __ATOMIC_RELAXED,
                          VR_AGENT);
     }
+  }
+  // The same payload to M sinks (the owner's gather), and M payloads to M sinks
+  // (a scatter): the flag travels inside every message, nothing to batch.
+  template <int M>
+  static __device__ __forceinline__ void send_many(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg &v, uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v, flag, lane);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_each(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg (&v)[M], uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v[i], flag, lane);
   }
   // watch_first: the message is expected to be still on its way, so start by
   // watching its last flag word instead of reading the whole message in vain.
@@ -249,6 +264,7 @@ template <int U, int DT>
 struct WireLL16 {
   static constexpr uint32_t kWireBytes = 64u * 8u * U;    // payload one wave moves per step
   static constexpr uint32_t kSlotBytes = 64u * 16u * U;   // message bytes in the sink
+  static constexpr bool kBatchSends = false;   // the flag travels inside every message
   static constexpr int kAuxAgent = 16;                             // sc1
   static constexpr int kAuxAgentVolatile = (int)0x80000010u;       // sc1, never hoisted or merged
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -296,6 +312,20 @@ struct WireLL16 {
       const u32x4 msg = {v.d[u][0], v.d[u][1], flag, flag};
       __builtin_amdgcn_raw_buffer_store_b128(msg, rs, (u * 64u + lane) * 16u, 0, kAuxAgent);
     }
+  }
+  // The same payload to M sinks (the owner's gather), and M payloads to M sinks
+  // (a scatter): the flag travels inside every message, nothing to batch.
+  template <int M>
+  static __device__ __forceinline__ void send_many(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg &v, uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v, flag, lane);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_each(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg (&v)[M], uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v[i], flag, lane);
   }
   // watch_first: the message is expected to be still on its way, so start by
   // watching its last flag word instead of reading the whole message in vain.
@@ -360,6 +390,7 @@ template <int U, int DT>
 struct WireRt128 {
   static constexpr uint32_t kWireBytes = 480u * U;
   static constexpr uint32_t kSlotBytes = 512u * U;
+  static constexpr bool kBatchSends = false;   // the flag travels inside every message
   struct Reg {
     uint32_t d[U][2];
   };
@@ -407,6 +438,20 @@ struct WireRt128 {
       __hip_atomic_store(reinterpret_cast<uint64_t *>(slot) + u * 64 + lane, (uint64_t)x | ((uint64_t)y << 32),
                          __ATOMIC_RELAXED, VR_AGENT);
     }
+  }
+  // The same payload to M sinks (the owner's gather), and M payloads to M sinks
+  // (a scatter): the flag travels inside every message, nothing to batch.
+  template <int M>
+  static __device__ __forceinline__ void send_many(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg &v, uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v, flag, lane);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_each(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg (&v)[M], uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v[i], flag, lane);
   }
   // All loads of a poll are issued before any of them is looked at, so that a
   // poll costs one memory round trip however many messages it covers.
@@ -477,6 +522,7 @@ template <int U, int DT>
 struct WireRt256 {
   static constexpr uint32_t kWireBytes = 960u * U;
   static constexpr uint32_t kSlotBytes = 1024u * U;
+  static constexpr bool kBatchSends = false;   // the flag travels inside every message
   static constexpr int kAuxAgent = 16;                             // sc1
   static constexpr int kAuxAgentVolatile = (int)0x80000010u;       // sc1, never hoisted or merged
   struct Reg {
@@ -544,6 +590,20 @@ struct WireRt256 {
     v.d[u][3] = l == 3u ? b3 : l == 7u ? b7 : l == 11u ? b11 : msg.w;
     return ((l & 3u) != 3u) | (msg.w == flag);
   }
+  // The same payload to M sinks (the owner's gather), and M payloads to M sinks
+  // (a scatter): the flag travels inside every message, nothing to batch.
+  template <int M>
+  static __device__ __forceinline__ void send_many(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg &v, uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v, flag, lane);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_each(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg (&v)[M], uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) send(slot[i], fw[i], v[i], flag, lane);
+  }
   // watch_first: the message is expected to be still on its way, so start by
   // watching its last flag word instead of reading the whole message in vain.
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *, Reg &v,
@@ -591,15 +651,32 @@ struct WireRt256 {
 };
 
 // Flag-word format: full 16-byte-per-lane payload lines plus ONE flag word per
-// message in a separate array, ordered by agent-scope fences: the sender stores
-// the payload, executes a release fence (L2 write-back), then lane 0 stores the
-// flag; the receiver polls the flag word and executes an acquire fence (cache
-// invalidate) before it loads the payload.  Assumes nothing about store
-// atomicity, and pays two cache-maintenance operations per message for it.
-template <int U, typename V, int DT>
+// message in a separate array.  Three ways to order payload and flag:
+//   FLAG_FENCE        the sender stores the payload, executes an agent-scope release
+//                     fence (buffer_wbl2: L2 write-back), then stores the flag; the
+//                     receiver polls the flag word and executes an acquire fence
+//                     (buffer_inv: cache invalidate) before it loads the payload.
+//                     Assumes nothing beyond the HIP memory model and pays two
+//                     cache-maintenance operations per synchronisation for it.
+//   FLAG_FENCE_WT     the same fences, payload stored written through at agent scope
+//                     (sc1), so the release finds nothing dirty to write back.
+//   FLAG_SCOPED       every access at agent scope and no cache maintenance: payload
+//                     stores are written through (sc1), the sender waits until they
+//                     have completed (s_waitcnt vmcnt(0)) before it stores the flag;
+//                     the receiver polls the flag and then loads the payload with
+//                     agent-scope loads (sc1), which never hit a stale line.
+// A wave that owes several messages at once stores all payloads, synchronises
+// ONCE, then stores all flags (send_many / send_each); a wave that waits for
+// several polls all flag words and synchronises once (recv_many).
+enum FlagSync : int { FLAG_FENCE = 0, FLAG_FENCE_WT = 1, FLAG_SCOPED = 2 };
+
+template <int U, typename V, int DT, int SYNC>
 struct WireFlag {
   static constexpr uint32_t kWireBytes = 64u * (uint32_t)sizeof(V) * U;
   static constexpr uint32_t kSlotBytes = kWireBytes;
+  static constexpr bool kBatchSends = true;
+  static constexpr int kAuxAgent = 16;                             // sc1
+  static constexpr int kAuxAgentVolatile = (int)0x80000010u;       // sc1, never hoisted or merged
   struct Reg {
     V d[U];
   };
@@ -629,12 +706,81 @@ struct WireFlag {
 #pragma unroll
     for (int u = 0; u < U; ++u) v.d[u] = vadd<DT>(m.d[u], v.d[u]);
   }
+
+  // Payload of one message into its slot; not yet announced.
+  static __device__ __forceinline__ void put(char *slot, const Reg &v, uint32_t lane) {
+    if constexpr (SYNC == FLAG_FENCE) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) reinterpret_cast<V *>(slot)[u * 64 + lane] = v.d[u];
+    } else {
+      const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot, kSlotBytes);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
+        if constexpr (sizeof(V) == 16)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(io_u32x4, v.d[u]), rs, off, 0, kAuxAgent);
+        else
+          __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(io_u32x2, v.d[u]), rs, off, 0, kAuxAgent);
+      }
+    }
+  }
+  // Everything put so far is visible at agent scope once this returns.
+  static __device__ __forceinline__ void publish() {
+    if constexpr (SYNC == FLAG_SCOPED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  }
+  // After the flags have been seen: what the senders published may be loaded.
+  static __device__ __forceinline__ void subscribe() {
+    if constexpr (SYNC == FLAG_SCOPED) asm volatile("" ::: "memory");
+    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  static __device__ __forceinline__ void get(const char *slot, Reg &v, uint32_t lane) {
+    if constexpr (SYNC == FLAG_SCOPED) {
+      const __amdgpu_buffer_rsrc_t rs = wave_rsrc(slot, kSlotBytes);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t off = (u * 64u + lane) * (uint32_t)sizeof(V);
+        if constexpr (sizeof(V) == 16)
+          v.d[u] = __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kAuxAgentVolatile));
+        else
+          v.d[u] = __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kAuxAgentVolatile));
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) v.d[u] = reinterpret_cast<const V *>(slot)[u * 64 + lane];
+    }
+  }
+  // Lane i < M stores the flag of message i.
+  template <int M>
+  static __device__ __forceinline__ void raise(uint32_t *const (&fw)[M], uint32_t flag, uint32_t lane) {
+    static_assert(M <= 64, "one lane per flag word");
+    uint32_t *mine = fw[0];
+#pragma unroll
+    for (int i = 1; i < M; ++i) mine = lane == (uint32_t)i ? fw[i] : mine;
+    if (lane < (uint32_t)M) __hip_atomic_store(mine, flag, __ATOMIC_RELAXED, VR_AGENT);
+  }
+
   static __device__ __forceinline__ void send(char *slot, uint32_t *flagword, const Reg &v,
                                               uint32_t flag, uint32_t lane) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) reinterpret_cast<V *>(slot)[u * 64 + lane] = v.d[u];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    put(slot, v, lane);
+    publish();
     if (lane == 0) __hip_atomic_store(flagword, flag, __ATOMIC_RELAXED, VR_AGENT);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_many(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg &v, uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) put(slot[i], v, lane);
+    publish();
+    raise<M>(fw, flag, lane);
+  }
+  template <int M>
+  static __device__ __forceinline__ void send_each(char *const (&slot)[M], uint32_t *const (&fw)[M],
+                                                   const Reg (&v)[M], uint32_t flag, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < M; ++i) put(slot[i], v[i], lane);
+    publish();
+    raise<M>(fw, flag, lane);
   }
   static __device__ __forceinline__ bool recv(const char *slot, const uint32_t *flagword, Reg &v,
                                               uint32_t flag, uint32_t lane, Spin &spin,
@@ -645,12 +791,11 @@ struct WireFlag {
     while (__hip_atomic_load(flagword, __ATOMIC_RELAXED, VR_AGENT) != flag) {
       if (spin.give_up(polls)) return false;
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-#pragma unroll
-    for (int u = 0; u < U; ++u) v.d[u] = reinterpret_cast<const V *>(slot)[u * 64 + lane];
+    subscribe();
+    get(slot, v, lane);
     return true;
   }
-  // M messages: wait for every flag word, ONE acquire fence, then all payloads.
+  // M messages: wait for every flag word, synchronise ONCE, then all payloads.
   template <int M>
   static __device__ __forceinline__ bool recv_many(const char *const (&slot)[M],
                                                    const uint32_t *const (&flagword)[M], Reg (&v)[M],
@@ -665,11 +810,9 @@ struct WireFlag {
       if (ok) break;                       // same words in every lane: wave-uniform
       if (spin.give_up(polls)) return false;
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    subscribe();
 #pragma unroll
-    for (int i = 0; i < M; ++i)
-#pragma unroll
-      for (int u = 0; u < U; ++u) v[i].d[u] = reinterpret_cast<const V *>(slot[i])[u * 64 + lane];
+    for (int i = 0; i < M; ++i) get(slot[i], v[i], lane);
     return true;
   }
 };
@@ -694,13 +837,15 @@ struct Sinks {
   }
 };
 
-// Rank and wire of this wave.  A launch either holds every rank's work-groups
-// (block b belongs to rank b % N) or one rank's only (solo_rank).
+// Rank and wire of this wave.  A launch holds the work-groups of the ranks
+// [rank_first, rank_first + rank_count): all N of them (block b belongs to rank
+// b % N), one rank only, or any group in between; block b belongs to rank
+// rank_first + b % rank_count.
 #define VR_WAVE_PROLOGUE                                                             \
-  const bool solo = a.solo_rank >= 0;                                                \
-  const int r = solo ? a.solo_rank : (int)(blockIdx.x % N);                          \
+  const uint32_t held = (uint32_t)a.rank_count;                                      \
+  const int r = a.rank_first + (int)(blockIdx.x % held);                             \
   const uint32_t lane = threadIdx.x & 63u;                                           \
-  const uint32_t wid = (solo ? blockIdx.x : blockIdx.x / N) * (blockDim.x >> 6) + (threadIdx.x >> 6); \
+  const uint32_t wid = (blockIdx.x / held) * (blockDim.x >> 6) + (threadIdx.x >> 6); \
   if (wid >= a.waves_per_rank) return;                                               \
   Spin spin{a.spin_limit, a.status, lane, false};                                    \
   const bool nt = a.stream_io != 0;                                                  \
@@ -769,10 +914,15 @@ __global__ __launch_bounds__(256) void k_wire_parallel(WireArgs a) {
 #pragma unroll
       for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);    // peers in order rank+1, rank+2, ...
       const uint32_t mine = wl::parallel_slot(x_id, r, s);
+      char *gs[N - 1];
+      uint32_t *gf[N - 1];
+#pragma unroll
       for (int i = 0; i < N - 1; ++i) {
         const int next = (r + i + 1) % N;
-        W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
+        gs[i] = sk.gath(next, mine);
+        gf[i] = sk.gflag(next, mine);
       }
+      W::template send_many<N - 1>(gs, gf, v, flag, lane);
       W::store(dst + off, left, lane, v, nt);
     }
   }
@@ -793,10 +943,25 @@ __global__ __launch_bounds__(256) void k_wire_sequential(WireArgs a) {
     const uint32_t flag = a.seq + t / NSLOT, s = t % NSLOT;
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
     const uint32_t mine = wl::ring_slot(wpr, r, wid, s);
-    for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
-      W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
+    if constexpr (W::kBatchSends) {
+      // all N - 1 scatters behind one synchronisation
+      char *ss[N - 1];
+      uint32_t *sf[N - 1];
+      typename W::Reg p[N - 1];
+#pragma unroll
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        p[i] = W::load(src + next * chunk + off, left, lane, nt);
+        ss[i] = sk.scat(next, mine);
+        sf[i] = sk.sflag(next, mine);
+      }
+      W::template send_each<N - 1>(ss, sf, p, flag, lane);
+    } else {
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
+        W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
+      }
     }
     typename W::Reg v = W::load(src + r * chunk + off, left, lane, nt);
     const char *ms[N - 1];
@@ -811,9 +976,16 @@ __global__ __launch_bounds__(256) void k_wire_sequential(WireArgs a) {
     W::template recv_many<N - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);      // peers in order rank+1, rank+2, ...
-    for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
+    {
+      char *gs[N - 1];
+      uint32_t *gf[N - 1];
+#pragma unroll
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        gs[i] = sk.gath(next, mine);
+        gf[i] = sk.gflag(next, mine);
+      }
+      W::template send_many<N - 1>(gs, gf, v, flag, lane);
     }
     W::store(dst + r * chunk + off, left, lane, v, nt);
 #pragma unroll
@@ -852,10 +1024,24 @@ __global__ __launch_bounds__(256) void k_wire_simple(WireArgs a) {
     const uint32_t flag = a.seq + (uint32_t)(message / kPerSection);   // seqNo + seqDelta
     const uint32_t left = bytes_left(chunk, off, W::kWireBytes);
     const uint32_t mine = wl::simple_slot(r, pos);
-    for (int i = 0; i < N - 1; ++i) {                             // scatter
-      const int next = (r + i + 1) % N;
-      const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
-      W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
+    if constexpr (W::kBatchSends) {                               // scatter, one synchronisation
+      char *ss[N - 1];
+      uint32_t *sf[N - 1];
+      typename W::Reg p[N - 1];
+#pragma unroll
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        p[i] = W::load(src + next * chunk + off, left, lane, nt);
+        ss[i] = sk.scat(next, mine);
+        sf[i] = sk.sflag(next, mine);
+      }
+      W::template send_each<N - 1>(ss, sf, p, flag, lane);
+    } else {
+      for (int i = 0; i < N - 1; ++i) {                           // scatter
+        const int next = (r + i + 1) % N;
+        const typename W::Reg p = W::load(src + next * chunk + off, left, lane, nt);
+        W::send(sk.scat(next, mine), sk.sflag(next, mine), p, flag, lane);
+      }
     }
     typename W::Reg v = W::load(src + r * chunk + off, left, lane, nt);    // pollRecvReduceBcast
     const char *ms[N - 1];
@@ -871,9 +1057,16 @@ __global__ __launch_bounds__(256) void k_wire_simple(WireArgs a) {
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) W::add(v, m[i]);
     W::store(dst + r * chunk + off, left, lane, v, nt);           // write back locally first
-    for (int i = 0; i < N - 1; ++i) {
-      const int next = (r + i + 1) % N;
-      W::send(sk.gath(next, mine), sk.gflag(next, mine), v, flag, lane);
+    {
+      char *gs[N - 1];
+      uint32_t *gf[N - 1];
+#pragma unroll
+      for (int i = 0; i < N - 1; ++i) {
+        const int next = (r + i + 1) % N;
+        gs[i] = sk.gath(next, mine);
+        gf[i] = sk.gflag(next, mine);
+      }
+      W::template send_many<N - 1>(gs, gf, v, flag, lane);
     }
 #pragma unroll
     for (int i = 0; i < N - 1; ++i) {                             // pollGatherOutputs
@@ -1044,14 +1237,23 @@ __global__ __launch_bounds__(256) void k_wire_bisect(WireArgs a) {
       W::template recv_many<B - 1>(ms, mf, m, flag, lane, spin);
 #pragma unroll
       for (int i = 0; i < B - 1; ++i) W::add(v, m[i]);    // pair sums in order l+1, l+2, ...
+      // gather to the same-parity ranks and forward to the pair (bisect_transmit.hpp:411-417)
       const uint32_t mine = wl::bisect_close_slot(wg, l, s);
+      const uint32_t far_out = wl::bisect_far_slot(wpr, B, wid, s);
+      char *gs[B];
+      uint32_t *gf[B];
+#pragma unroll
       for (int i = 0; i < B - 1; ++i) {
         const int nx = (r + i * 2 + 2) % N;
-        W::send(sk.gath(nx, mine), sk.gflag(nx, mine), v, flag, lane);
+        gs[i] = sk.gath(nx, mine);
+        gf[i] = sk.gflag(nx, mine);
       }
+      gs[B - 1] = sk.gath(pair, far_out);
+      gf[B - 1] = sk.gflag(pair, far_out);
+      W::template send_many<B>(gs, gf, v, flag, lane);
     }
     const uint32_t far = wl::bisect_far_slot(wpr, B, wid, s);
-    W::send(sk.gath(pair, far), sk.gflag(pair, far), v, flag, lane);
+    if ((int)y != l) W::send(sk.gath(pair, far), sk.gflag(pair, far), v, flag, lane);
     W::store(dst + close_off + off, left, lane, v, nt);
     {                                                 // pollFarGatherOutput
       typename W::Reg m;
@@ -1070,6 +1272,23 @@ __global__ void k_wire_clear(uint64_t *p, size_t n64) {
     p[i] = 0;
 }
 
+// Clears the first `slot_bytes` bytes (message slots) and the first `flag_bytes`
+// bytes at `flag_off` (flag words) of every rank's scatter and gather sink: what
+// one launch is about to use.  blockIdx.y picks the sink; all sizes are multiples
+// of 16.
+__global__ void k_wire_clear_sinks(PtrTable scatter, PtrTable gather, int nranks, size_t slot_bytes,
+                                   size_t flag_off, size_t flag_bytes) {
+  const int which = (int)blockIdx.y;
+  char *sink = static_cast<char *>(which < nranks ? scatter.p[which] : gather.p[which - nranks]);
+  const size_t n_slots = slot_bytes / 16, n_flags = flag_bytes / 16;
+  const io_u32x4 zero = {0u, 0u, 0u, 0u};
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_slots + n_flags;
+       i += (size_t)gridDim.x * blockDim.x) {
+    io_u32x4 *p = reinterpret_cast<io_u32x4 *>(i < n_slots ? sink + i * 16 : sink + flag_off + (i - n_slots) * 16);
+    *p = zero;
+  }
+}
+
 // Messages per lane and step for each format; every slot stays within 2 KiB.
 constexpr int kUnrollLL = 4;     // 1 KiB payload in a 2 KiB message
 constexpr int kUnrollLL16 = 2;   // 1 KiB payload in a 2 KiB message
@@ -1081,14 +1300,14 @@ static_assert(WireLL<kUnrollLL, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot 
 static_assert(WireLL16<kUnrollLL16, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 static_assert(WireRt128<kUnrollRt128, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 static_assert(WireRt256<kUnrollRt256, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
-static_assert(WireFlag<kUnrollFlag, h8, DT_F16>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
+static_assert(WireFlag<kUnrollFlag, h8, DT_F16, FLAG_FENCE>::kSlotBytes <= wl::kSlotBytesMax, "slot too large");
 
 // ---- the library's own scratch -----------------------------------------------------------
 // Fixed region for the entry point that must not allocate: every rank's scatter
 // and gather sink for up to kStaticMaxRanks ranks of kStaticWiresPerRank wires
-// (no SimpleTransmit sections), then 256 bytes that hold the status word.  In
-// host code the array's name is only a handle: its device address is looked up
-// once per device with hipGetSymbolAddress.
+// (no SimpleTransmit sections), padded by 256 bytes.  In host code the array's
+// name is only a handle: its device address is looked up once per device with
+// hipGetSymbolAddress.
 constexpr size_t kStaticScratchBytes =
     (size_t)kStaticMaxRanks * wl::layout_for(kStaticMaxRanks, kStaticWiresPerRank, false).rank_bytes + 256;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
@@ -1155,9 +1374,15 @@ static const void *wire_kernel_dt(WireFlow flow, WireFormat fmt, int vec_halves,
     case WIRE_FMT_RT128: return flow_kernel<WireRt128<kUnrollRt128, DT>>(flow, nranks);
     case WIRE_FMT_RT256: return flow_kernel<WireRt256<kUnrollRt256, DT>>(flow, nranks);
     case WIRE_FMT_LL16: return flow_kernel<WireLL16<kUnrollLL16, DT>>(flow, nranks);
+    case WIRE_FMT_FLAG_WT:
+      return vec_halves == 8 ? flow_kernel<WireFlag<kUnrollFlag, h8, DT, FLAG_FENCE_WT>>(flow, nranks)
+                             : flow_kernel<WireFlag<kUnrollFlag, h4, DT, FLAG_FENCE_WT>>(flow, nranks);
+    case WIRE_FMT_FLAG_SCOPED:
+      return vec_halves == 8 ? flow_kernel<WireFlag<kUnrollFlag, h8, DT, FLAG_SCOPED>>(flow, nranks)
+                             : flow_kernel<WireFlag<kUnrollFlag, h4, DT, FLAG_SCOPED>>(flow, nranks);
     default:
-      return vec_halves == 8 ? flow_kernel<WireFlag<kUnrollFlag, h8, DT>>(flow, nranks)
-                             : flow_kernel<WireFlag<kUnrollFlag, h4, DT>>(flow, nranks);
+      return vec_halves == 8 ? flow_kernel<WireFlag<kUnrollFlag, h8, DT, FLAG_FENCE>>(flow, nranks)
+                             : flow_kernel<WireFlag<kUnrollFlag, h4, DT, FLAG_FENCE>>(flow, nranks);
   }
 }
 
@@ -1172,9 +1397,21 @@ uint32_t wire_bytes_per_step(WireFormat fmt, int vec_halves) {
     case WIRE_FMT_RT128: return WireRt128<kUnrollRt128, DT_F16>::kWireBytes;
     case WIRE_FMT_RT256: return WireRt256<kUnrollRt256, DT_F16>::kWireBytes;
     case WIRE_FMT_LL16: return WireLL16<kUnrollLL16, DT_F16>::kWireBytes;
+    default:   // the three flag-word variants move the same wires
+      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16, FLAG_FENCE>::kWireBytes
+                             : WireFlag<kUnrollFlag, h4, DT_F16, FLAG_FENCE>::kWireBytes;
+  }
+}
+
+uint32_t wire_slot_bytes(WireFormat fmt, int vec_halves) {
+  switch (fmt) {
+    case WIRE_FMT_LL: return WireLL<kUnrollLL, DT_F16>::kSlotBytes;
+    case WIRE_FMT_RT128: return WireRt128<kUnrollRt128, DT_F16>::kSlotBytes;
+    case WIRE_FMT_RT256: return WireRt256<kUnrollRt256, DT_F16>::kSlotBytes;
+    case WIRE_FMT_LL16: return WireLL16<kUnrollLL16, DT_F16>::kSlotBytes;
     default:
-      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16>::kWireBytes
-                             : WireFlag<kUnrollFlag, h4, DT_F16>::kWireBytes;
+      return vec_halves == 8 ? WireFlag<kUnrollFlag, h8, DT_F16, FLAG_FENCE>::kSlotBytes
+                             : WireFlag<kUnrollFlag, h4, DT_F16, FLAG_FENCE>::kSlotBytes;
   }
 }
 
@@ -1217,6 +1454,20 @@ hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_hal
   const dim3 grid(blocks), block(block_threads);
   if (cooperative) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
   return hipLaunchKernel(fn, grid, block, kargs, 0, s);
+}
+
+hipError_t launch_wire_clear_sinks(hipStream_t s, const PtrTable &scatter, const PtrTable &gather, int nranks,
+                                   size_t slot_bytes, size_t flag_off, size_t flag_bytes) {
+  slot_bytes = (slot_bytes + 15) / 16 * 16;
+  flag_bytes = (flag_bytes + 15) / 16 * 16;
+  if (flag_off % 16) return hipErrorInvalidValue;
+  const size_t per_sink = (slot_bytes + flag_bytes) / 16;
+  if (per_sink == 0) return hipSuccess;
+  size_t bx = (per_sink + 255) / 256;
+  if (bx > 64) bx = 64;
+  hipLaunchKernelGGL(k_wire_clear_sinks, dim3((uint32_t)bx, 2u * (uint32_t)nranks), dim3(256), 0, s, scatter,
+                     gather, nranks, slot_bytes, flag_off, flag_bytes);
+  return hipGetLastError();
 }
 
 hipError_t launch_wire_clear(hipStream_t s, void *p, size_t bytes) {

@@ -2,9 +2,12 @@
 // library's fixed region), launch sizing and sequence-number bookkeeping, the
 // one-rank entry points and the time-out check.  Kernels: vr_wire.hip.
 
+#include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <string>
+#include <unordered_map>
 
 #include "vr_host.h"
 
@@ -88,54 +91,70 @@ static int wire_clear(const WireSinks &k, int nranks, hipStream_t s) {
 
 struct WireLaunch {
   const WireSinks *sinks;
-  WireHistory *hist;      // null: the caller owns the sinks and the sequence numbers (one-rank launches)
+  WireHistory *hist;      // null: the caller owns the sinks and the sequence numbers (rank-group launches)
   uint32_t *status;
-  int solo_rank;          // >= 0: launch this rank's wires only
+  int first, count;       // the launch holds the wires of ranks [first, first + count)
   bool always_clear;      // clear the sinks before every launch (fixed scratch shared by contexts)
 };
 
-// Launches one wire-transport collective.  `user_wires` (0 = automatic) is the
-// number of sub-groups per rank a caller asked for with -g/-w.  *seq_io is the
-// first flag value the caller proposes; it is replaced by the one actually used
-// (it restarts from 1 when the 32-bit counter would wrap through 0).  Returns
-// through *flags_used how many consecutive flag values the launch consumes.
-static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
-                       const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t *seq_io,
-                       uint32_t user_wires, uint32_t *flags_used, const WireLaunch &wlch) {
-  uint32_t seq = *seq_io;
-  if (seq == 0)
-    return fail(VR_ERR_INVALID, "sequence number 0 cannot be told from freshly zeroed scratch");
-  const WireSinks &k = *wlch.sinks;
-  const int N = c->nranks;
-  const WireFlow flow = a->wire_flow();
+// Wire format of an algo under the context's settings.  `vec_halves` = 8 says that
+// every pointer and the chunk allow 16-byte accesses.
+static WireFormat format_for(const vr_ctx *c, const AlgoInfo *a, size_t chunk_bytes, int vec_halves) {
   WireFormat fmt = a->wire_format();
   const bool big = fmt == WIRE_FMT_RT128 || fmt == WIRE_FMT_RT256;
   if (big && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
   // Self-validating 8-byte messages for the Rt64_128 families too: nothing beyond
   // 8-byte store atomicity is assumed, at half the payload per message.
   if (big && c->tune.wire_fenced == 2) fmt = WIRE_FMT_LL;
+  if (big && c->tune.wire_fenced == 3) fmt = WIRE_FMT_FLAG_WT;
+  if (big && c->tune.wire_fenced == 4) fmt = WIRE_FMT_FLAG_SCOPED;
   if (fmt == WIRE_FMT_LL16 && c->tune.wire_msg16 == 0) fmt = WIRE_FMT_LL;
-  if (flow == WIRE_SIMPLE && !k.simple_ok)
-    return fail(VR_ERR_INVALID, "these sinks have no room for SimpleTransmit's 2 MiB sender sections");
-  // The flag values of a launch are kernel arguments, and whether the sinks must
-  // be cleared first is decided here on the host: a captured launch would replay
-  // with stale flags.  (With always_clear every replay starts from clean sinks.)
-  if (!wlch.always_clear) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
-      return fail(VR_ERR_INVALID, "the wire transport cannot be captured into a graph: its flag values "
-                                  "are per-launch kernel arguments (capture the direct transport)");
-    (void)hipGetLastError();
-  }
   // `parallel` names the transmit, not a wire format: it takes the reference's
   // 256-byte messages (16 bytes per lane) when every pointer and the chunk allow
   // 16-byte accesses, its 128-byte messages otherwise.
   if (fmt == WIRE_FMT_RT128 && a == &kAlgos[VR_ALGO_PARALLEL] && vec_halves == 8 && chunk_bytes % 16 == 0)
     fmt = WIRE_FMT_RT256;
+  return fmt;
+}
+
+// Does the algo's wire format, as the context is set, move 16 bytes per lane when
+// the chunk allows it (and therefore need 16-byte aligned buffers then)?  The
+// 8-byte-message formats (Rt64, Rt64_128) and the 16-byte-message formats (whose
+// calcWorkSize already demands 16-byte alignment) do not depend on it.
+static bool format_widens_with_alignment(const vr_ctx *c, const AlgoInfo *a) {
+  if (a == &kAlgos[VR_ALGO_PARALLEL]) return true;
+  const WireFormat fmt = a->wire_format();
+  const bool big = fmt == WIRE_FMT_RT128 || fmt == WIRE_FMT_RT256;
+  return big && (c->tune.wire_fenced == 1 || c->tune.wire_fenced == 3 || c->tune.wire_fenced == 4);
+}
+
+// Shape of one wire-transport launch: which kernel, how many wires per rank, how
+// many loop steps and how many consecutive flag values it consumes.
+struct WirePlan {
+  WireFlow flow;
+  WireFormat fmt;
+  uint32_t wpr = 0;              // wires (waves) per rank; 0 = nothing to move
+  uint32_t blocks_per_rank = 0;
+  size_t steps = 0;
+  uint32_t flags_used = 0;
+};
+
+// `user_wires` (0 = automatic) is the number of sub-groups per rank a caller asked
+// for with -g/-w; `k` the sinks the launch will use.
+static int plan_wire(const vr_ctx *c, const AlgoInfo *a, size_t chunk_bytes, int vec_halves,
+                     uint32_t user_wires, const WireSinks &k, WirePlan *plan) {
+  const int N = c->nranks;
+  const WireFlow flow = a->wire_flow();
+  const WireFormat fmt = format_for(c, a, chunk_bytes, vec_halves);
+  *plan = WirePlan();
+  plan->flow = flow;
+  plan->fmt = fmt;
+  if (flow == WIRE_SIMPLE && !k.simple_ok)
+    return fail(VR_ERR_INVALID, "these sinks have no room for SimpleTransmit's 2 MiB sender sections");
   const uint32_t psg = flow == WIRE_PARALLEL ? (uint32_t)N : flow == WIRE_BISECT ? (uint32_t)N / 2 : 1u;
   const uint32_t waves_per_block = kWireBlockThreads / 64;
-  // Every wave may wait for any other: keep the grid (for one-rank launches: the N
-  // grids together) within what the device holds at once.
+  // Every wave may wait for any other: keep the grid (for rank-group launches: the
+  // groups' grids together) within what the device holds at once.
   int per_cu = 0;
   if (hipError_t e = wire_blocks_per_cu(flow, fmt, vec_halves, N, kWireBlockThreads, c->dtype, &per_cu))
     return fail_hip(e, "occupancy query");
@@ -145,7 +164,7 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   if (wpr_limit < psg) return fail(VR_ERR_INVALID, "sinks or device too small for this rank count");
   const uint32_t wire_bytes = wire_bytes_per_step(fmt, vec_halves);
   const size_t wires_per_chunk = div_up(chunk_bytes, wire_bytes);
-  if (wires_per_chunk == 0) { *flags_used = 0; return VR_OK; }
+  if (wires_per_chunk == 0) return VR_OK;
   size_t want = user_wires ? (size_t)user_wires / psg * psg : wires_per_chunk * psg;
   if (want < psg) want = psg;
   if (want > wpr_limit) want = wpr_limit;
@@ -161,11 +180,44 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   const uint32_t wpr = (uint32_t)want;
   if (wl::slots_needed((int)flow, N, wpr) > k.layout.slots)
     return fail(VR_ERR_INVALID, "internal: sink smaller than the flow's slot range");
-  const uint32_t blocks_per_rank = (uint32_t)div_up(wpr, waves_per_block);
-  const size_t steps = div_up(wires_per_chunk, wpr / psg);
+  plan->wpr = wpr;
+  plan->blocks_per_rank = (uint32_t)div_up(wpr, waves_per_block);
+  plan->steps = div_up(wires_per_chunk, wpr / psg);
   const uint32_t nslot_min = 4;
-  *flags_used = flow == WIRE_SIMPLE ? (uint32_t)(steps * wpr / wl::kSimplePerSection + 1)
-                                    : (uint32_t)((steps - 1) / nslot_min + 1);
+  plan->flags_used = flow == WIRE_SIMPLE ? (uint32_t)(plan->steps * wpr / wl::kSimplePerSection + 1)
+                                         : (uint32_t)((plan->steps - 1) / nslot_min + 1);
+  return VR_OK;
+}
+
+// Launches one wire-transport collective.  *seq_io is the first flag value the
+// caller proposes; it is replaced by the one actually used (it restarts from 1
+// when the 32-bit counter would wrap through 0).  Returns through *flags_used how
+// many consecutive flag values the launch consumes.
+static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable &in,
+                       const PtrTable &out, size_t chunk_bytes, int vec_halves, uint32_t *seq_io,
+                       uint32_t user_wires, uint32_t *flags_used, const WireLaunch &wlch) {
+  uint32_t seq = *seq_io;
+  if (seq == 0)
+    return fail(VR_ERR_INVALID, "sequence number 0 cannot be told from freshly zeroed scratch");
+  const WireSinks &k = *wlch.sinks;
+  const int N = c->nranks;
+  // The flag values of a launch are kernel arguments, and whether the sinks must
+  // be cleared first is decided here on the host: a captured launch would replay
+  // with stale flags.  (With always_clear every replay starts from clean sinks.)
+  if (!wlch.always_clear) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(VR_ERR_INVALID, "the wire transport cannot be captured into a graph: its flag values "
+                                  "are per-launch kernel arguments (capture the direct transport)");
+    (void)hipGetLastError();
+  }
+  WirePlan plan;
+  if (int rc = plan_wire(c, a, chunk_bytes, vec_halves, user_wires, k, &plan)) return rc;
+  *flags_used = plan.flags_used;
+  if (plan.wpr == 0) return VR_OK;
+  const WireFlow flow = plan.flow;
+  const WireFormat fmt = plan.fmt;
+  const uint32_t wpr = plan.wpr, blocks_per_rank = plan.blocks_per_rank;
 
   // Flags must strictly increase on every slot and never be 0 (the value of
   // cleared scratch); a different flow or format re-interprets the sinks.  In all
@@ -176,7 +228,19 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
                                 "and restart from 1");
   if (wraps) seq = 1;
   if (wlch.always_clear) {
-    if (int rc = wire_clear(k, N, s)) return rc;
+    // only what this launch will index: its slot range and, for the flag-word
+    // formats, the flag words of those slots
+    PtrTable sc, ga;
+    memset(&sc, 0, sizeof sc);
+    memset(&ga, 0, sizeof ga);
+    for (int r = 0; r < N; ++r) {
+      sc.p[r] = k.scatter[r];
+      ga.p[r] = k.gather[r];
+    }
+    const size_t slots = wl::slots_needed((int)flow, N, wpr);
+    const hipError_t e = launch_wire_clear_sinks(s, sc, ga, N, slots * wire_slot_bytes(fmt, vec_halves),
+                                                 k.layout.flag_off, wire_fmt_is_flag(fmt) ? slots * 4 : 0);
+    if (e != hipSuccess) return fail_hip(e, "launch_wire_clear_sinks");
   } else if (wlch.hist) {
     WireHistory &h = *wlch.hist;
     const bool moved_back = h.used && (int32_t)(seq - h.next_min_seq) < 0;
@@ -203,7 +267,8 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
   args.status = wlch.status;
   args.ahead = c->tune.wire_ahead > 0 ? (uint32_t)c->tune.wire_ahead : kWireAhead;
-  args.solo_rank = wlch.solo_rank;
+  args.rank_first = wlch.first;
+  args.rank_count = wlch.count;
   // Inputs and outputs that cannot stay in the 256 MiB memory-side cache anyway are
   // streamed past it, which leaves that cache to the sinks (measured: faster from
   // 256 MiB of inputs + outputs on, slower below).
@@ -211,12 +276,11 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
                                        : 2 * (size_t)N * chunk_bytes * (size_t)N;     // N chunks per rank, in + out
   args.stream_io = c->tune.wire_stream_io >= 0 ? (uint32_t)c->tune.wire_stream_io
                                                : (io_bytes >= (256ull << 20) ? 1u : 0u);
-  const bool solo = wlch.solo_rank >= 0;
   // The grid is co-resident by construction; a cooperative launch (on request)
-  // lets the runtime check that once more.  One rank's launch cannot vouch for
-  // the other ranks' work-groups: always plain.
-  const bool cooperative = !solo && c->tune.wire_cooperative == 1;
-  const uint32_t blocks = solo ? blocks_per_rank : blocks_per_rank * (uint32_t)N;
+  // lets the runtime check that once more.  A launch that holds some of the ranks
+  // cannot vouch for the other ranks' work-groups: always plain.
+  const bool cooperative = wlch.count == N && c->tune.wire_cooperative == 1;
+  const uint32_t blocks = blocks_per_rank * (uint32_t)wlch.count;
   hipError_t e = launch_wire(s, flow, fmt, vec_halves, N, blocks, kWireBlockThreads, args,
                              cooperative, c->dtype);
   if (e != hipSuccess) return fail_hip(e, "launch_wire");
@@ -237,25 +301,24 @@ int wire_launch_ctx(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTable 
   if (!c->wire.ready)
     return fail(VR_ERR_INVALID, "the wire transport's scratch is not reserved: call "
                                 "vr_ctx_reserve_wire(ctx) once before the first wire-transport launch");
-  const WireLaunch wlch = {&c->wire.sinks, &c->wire.hist, c->status, -1, false};
+  const WireLaunch wlch = {&c->wire.sinks, &c->wire.hist, c->status, 0, c->nranks, false};
   return wire_launch(c, s, a, in, out, chunk_bytes, vec_halves, seq_io, user_wires, flags_used, wlch);
 }
 }  // namespace vr
 
 
-// The library's fixed scratch region on the context's device: its sinks (for the
-// context's rank count) and its status word.
-static int static_sinks(const vr_ctx *ctx, WireSinks *k, uint32_t **status) {
+// The library's fixed scratch region on the context's device, laid out as sinks
+// for the context's rank count.
+static int static_sinks(const vr_ctx *ctx, WireSinks *k) {
   void *fixed = nullptr;
   size_t bytes = 0;
   hipError_t e = wire_static_scratch(ctx->dev.device, &fixed, &bytes);
   if (e != hipSuccess) return fail_hip(e, "hipGetSymbolAddress(scratch)");
   const wl::Layout l = wl::layout_for(ctx->nranks, kStaticWiresPerRank, false);
-  if ((size_t)ctx->nranks * l.rank_bytes + 256 > bytes)
+  if ((size_t)ctx->nranks * l.rank_bytes > bytes)
     return fail(VR_ERR_INVALID, "the fixed scratch region holds at most " +
                                     std::to_string(kStaticMaxRanks) + " ranks");
   sinks_at(k, ctx->nranks, static_cast<char *>(fixed), l, kStaticWiresPerRank, false);
-  *status = reinterpret_cast<uint32_t *>(static_cast<char *>(fixed) + bytes - 256);
   return VR_OK;
 }
 
@@ -277,25 +340,23 @@ extern "C" int vr_allreduce_static(vr_ctx *ctx, void *stream, int algo, void *co
   if (p.a->wire_flow() == WIRE_SIMPLE)
     return fail(VR_ERR_INVALID, "vr_allreduce_static has no room for SimpleTransmit's 2 MiB sender sections");
   WireSinks k;
-  uint32_t *status = nullptr;
-  if (int rc = static_sinks(ctx, &k, &status)) return rc;
+  if (int rc = static_sinks(ctx, &k)) return rc;
   // The region is shared by every context on the device and keeps the last
-  // call's messages: every call clears the sinks first (a fill kernel on the
-  // stream), so the flags can start from 1 each time.
-  const WireLaunch wlch = {&k, nullptr, status, -1, true};
+  // call's messages: every call first clears the slots it is about to use (a
+  // fill kernel on the stream), so the flags can start from 1 each time.  The
+  // time-out word is the context's own, like that of its other wire launches.
+  const WireLaunch wlch = {&k, nullptr, ctx->status, 0, ctx->nranks, true};
   uint32_t seq = 1, used = 0;
-  ctx->static_used = true;
   return wire_launch(ctx, (hipStream_t)stream, p.a, p.in, p.out, p.chunk_elems * 2, p.vec_halves, &seq,
                      0, &used, wlch);
 }
 
-// Caller-owned sinks of a one-rank launch: the rank's own pair and its peers'.
-static int rank_sinks(const vr_ctx *ctx, int rank, void *scatter_buf, void *gather_buf,
-                      void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes, WireSinks *k) {
+// Caller-owned sinks of a rank-group launch: every rank's scatter and gather sink,
+// the launch's own ranks included.
+static int group_sinks(const vr_ctx *ctx, void *const peer_buf0[], void *const peer_buf1[],
+                       size_t sink_bytes, WireSinks *k) {
   const int N = ctx->nranks;
-  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
-  if (!scatter_buf || !gather_buf || !peer_buf0 || !peer_buf1)
-    return fail(VR_ERR_INVALID, "null scratch pointer");
+  if (!peer_buf0 || !peer_buf1) return fail(VR_ERR_INVALID, "null scratch pointer");
   const uint32_t wpr_max = wire_wpr_max(ctx);
   const wl::Layout l = wl::layout_for(N, wpr_max, true);
   if (sink_bytes < l.sink_bytes)
@@ -306,61 +367,196 @@ static int rank_sinks(const vr_ctx *ctx, int rank, void *scatter_buf, void *gath
   k->wpr_max = wpr_max;
   k->simple_ok = true;
   for (int r = 0; r < N; ++r) {
-    k->scatter[r] = r == rank ? scatter_buf : peer_buf0[r];
-    k->gather[r] = r == rank ? gather_buf : peer_buf1[r];
-    if (!k->scatter[r] || !k->gather[r]) return fail(VR_ERR_INVALID, "null peer sink for rank " + std::to_string(r));
+    k->scatter[r] = peer_buf0[r];
+    k->gather[r] = peer_buf1[r];
+    if (!k->scatter[r] || !k->gather[r]) return fail(VR_ERR_INVALID, "null sink for rank " + std::to_string(r));
     if ((uintptr_t)k->scatter[r] % 16 || (uintptr_t)k->gather[r] % 16)
       return fail(VR_ERR_UNALIGNED, "sinks must be 16-byte aligned");
   }
   return VR_OK;
 }
 
-// One rank of an all-reduce, the form the reference constructs per process
-// (allreduce.hpp:18-28, parallel_transmit.hpp:36-60, bisect_transmit.hpp:427-482).
-static int allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
-                          void *scatter_buf, void *gather_buf, void *const peer_buf0[],
-                          void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no,
-                          uint32_t user_wires) {
+// The launches that form one collective against caller-owned sinks wait for each
+// other, so their kernels must run at the same time.  Inside one process that
+// takes one hardware queue per launch: two launches on one stream run one after
+// the other, and a process has only a few hardware queues (GPU_MAX_HW_QUEUES, 4
+// unless the environment says otherwise) which further streams share.  Both would
+// end in a poll time-out; they are refused here instead, with the remedy.  A
+// collective is recognised by its sinks (rank 0's scatter sink) and its sequence
+// number, which every one of its launches must pass alike.
+namespace {
+struct GroupLaunches {
+  uint32_t seq = 0;
+  int nranks = 0;
+  void *stream_of[VR_MAX_RANKS] = {};
+  bool launched[VR_MAX_RANKS] = {};
+};
+std::mutex g_groups_lock;
+std::unordered_map<const void *, GroupLaunches> g_groups;
+
+int hardware_queues() {
+  const char *env = getenv("GPU_MAX_HW_QUEUES");
+  const int v = env ? atoi(env) : 0;
+  return v > 0 ? v : 4;
+}
+}  // namespace
+
+static int admit_group_launch(const vr_ctx *ctx, const void *family, void *stream, int first, int count,
+                              uint32_t seq) {
+  const int N = ctx->nranks;
+  if (count == N) return VR_OK;
+  std::lock_guard<std::mutex> hold(g_groups_lock);
+  GroupLaunches &g = g_groups[family];
+  if (g.seq != seq || g.nranks != N) {
+    g = GroupLaunches();
+    g.seq = seq;
+    g.nranks = N;
+  }
+  int streams = 0;
+  void *seen[VR_MAX_RANKS];
+  for (int r = 0; r < N; ++r) {
+    if (!g.launched[r] || (r >= first && r < first + count)) continue;
+    if (g.stream_of[r] == stream)
+      return fail(VR_ERR_INVALID, "ranks " + std::to_string(first) + ".." + std::to_string(first + count - 1) +
+                                      " and rank " + std::to_string(r) + " of one collective were launched on the "
+                                      "same stream: their kernels wait for each other and must run at the same "
+                                      "time (one stream per launch, or one vr_allreduce_ranks launch for both)");
+    bool known = false;
+    for (int i = 0; i < streams; ++i) known = known || seen[i] == g.stream_of[r];
+    if (!known) seen[streams++] = g.stream_of[r];
+  }
+  const int limit = hardware_queues();
+  if (streams + 1 > limit)
+    return fail(VR_ERR_INVALID, "this collective would need " + std::to_string(streams + 1) +
+                                    " concurrent launches from one process, which has " + std::to_string(limit) +
+                                    " hardware queues (GPU_MAX_HW_QUEUES): hold several ranks per launch with "
+                                    "vr_allreduce_ranks, or run the ranks in separate processes");
+  for (int r = first; r < first + count; ++r) {
+    g.launched[r] = true;
+    g.stream_of[r] = stream;
+  }
+  return VR_OK;
+}
+
+// Ranks [first, first + count) of an all-reduce, the form the reference constructs
+// once per process for one rank (allreduce.hpp:18-28, parallel_transmit.hpp:36-60,
+// bisect_transmit.hpp:427-482).
+static int allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first, int count,
+                           void *const inputs[], void *const outputs[], void *const peer_buf0[],
+                           void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no,
+                           uint32_t user_wires) {
   if (int rc = use_device(ctx)) return rc;
   const AlgoInfo *a = algo_info(algo);
   if (!a || a->allgather) return fail(VR_ERR_ALGO, "not an all-reduce algo");
   const int N = ctx->nranks;
-  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
-  if (!seq_no) return fail(VR_ERR_INVALID, "a one-rank launch needs the caller's sequence number");
-  if (!output) output = input;
-  // calcWorkSize sees this rank's pointers only (allreduce.hpp:108-122).
-  const void *table[VR_MAX_RANKS];
-  for (int r = 0; r < N; ++r) table[r] = input;
-  size_t work = 0;
-  if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
-  for (int r = 0; r < N; ++r) table[r] = output;
-  if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
-  if (ranges_partially_overlap(output, input, nelems * 2))
-    return fail(VR_ERR_OVERLAP, "output partially overlaps input");
-  WireSinks k;
-  if (int rc = rank_sinks(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
+  if (first < 0 || count < 1 || first + count > N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!inputs) return fail(VR_ERR_INVALID, "null input table");
+  if (!seq_no) return fail(VR_ERR_INVALID, "a rank-group launch needs the caller's sequence number");
+  // Every rank must pick the same message shape, so the access width may depend on
+  // nothing but the algo, the context's settings and the element count.  Formats
+  // that move 16 bytes per lane when the chunk is a multiple of 16 bytes then need
+  // 16-byte aligned buffers on every rank; the others accept what calcWorkSize
+  // accepts (allreduce.hpp:108-122).
+  const bool widens = format_widens_with_alignment(ctx, a);
   PtrTable in, out;
   memset(&in, 0, sizeof in);
   memset(&out, 0, sizeof out);
-  in.p[rank] = input;
-  out.p[rank] = output;
-  const size_t chunk_elems = work / 2;
-  // Every rank must pick the same message shape, so the access width may depend on
-  // nothing but the element count: 16-byte accesses whenever the chunk is a
-  // multiple of 16 bytes, and then this rank's buffers must allow them.
-  const int vec_halves = chunk_elems % 8 == 0 ? 8 : 4;
-  if (vec_halves == 8 && ((uintptr_t)input % 16 || (uintptr_t)output % 16))
-    return fail(VR_ERR_UNALIGNED, "one-rank launches move a chunk that is a multiple of 16 bytes with 16-byte "
-                                  "accesses on every rank: input and output must be 16-byte aligned");
+  size_t work = 0;
+  int vec_halves = a->msg_bytes == 16 ? 8 : 4;
+  for (int i = 0; i < count; ++i) {
+    void *input = inputs[i], *output = outputs && outputs[i] ? outputs[i] : inputs[i];
+    // calcWorkSize sees one rank's pointers at a time
+    const void *table[VR_MAX_RANKS];
+    for (int r = 0; r < N; ++r) table[r] = input;
+    if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
+    for (int r = 0; r < N; ++r) table[r] = output;
+    if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
+    if (ranges_partially_overlap(output, input, nelems * 2))
+      return fail(VR_ERR_OVERLAP, "output partially overlaps input");
+    if (widens && (work / 2) % 8 == 0) {
+      vec_halves = 8;
+      if ((uintptr_t)input % 16 || (uintptr_t)output % 16)
+        return fail(VR_ERR_UNALIGNED, std::string(a->name) + " moves a chunk that is a multiple of 16 bytes with "
+                                          "16-byte accesses on every rank: input and output must be 16-byte aligned");
+    }
+    in.p[first + i] = input;
+    out.p[first + i] = output;
+  }
+  WireSinks k;
+  if (int rc = group_sinks(ctx, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
   vr_geometry geom;
   if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
-  const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};
+  if (int rc = admit_group_launch(ctx, k.scatter[0], stream, first, count, *seq_no)) return rc;
+  const WireLaunch wlch = {&k, nullptr, ctx->status, first, count, false};
   uint32_t seq = *seq_no, used = 0;
-  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, chunk_elems * 2, vec_halves, &seq,
-                           user_wires, &used, wlch))
+  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, work, vec_halves, &seq, user_wires, &used,
+                           wlch))
     return rc;
   *seq_no = seq + (used > geom.steps ? used : geom.steps);
   if (*seq_no == 0) *seq_no = 1;
+  return VR_OK;
+}
+
+// The reference's one-rank parameter list: the rank's own sinks beside the peers'.
+static int one_rank_tables(const vr_ctx *ctx, int rank, void *scatter_buf, void *gather_buf,
+                           void *const peer_buf0[], void *const peer_buf1[], void *p0[], void *p1[]) {
+  const int N = ctx ? ctx->nranks : 0;
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!scatter_buf || !gather_buf || !peer_buf0 || !peer_buf1)
+    return fail(VR_ERR_INVALID, "null scratch pointer");
+  for (int r = 0; r < N; ++r) {
+    p0[r] = r == rank ? scatter_buf : peer_buf0[r];
+    p1[r] = r == rank ? gather_buf : peer_buf1[r];
+  }
+  return VR_OK;
+}
+
+static int check_grid(uint32_t groups, uint32_t subgroups, uint32_t simd, uint32_t *wires) {
+  // main.cpp:289-291, then allreduce.cpp:852/917.
+  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
+  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
+  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
+  const uint64_t w = (uint64_t)groups * subgroups;
+  *wires = w > 0xffffffffull ? 0xffffffffu : (uint32_t)w;
+  return VR_OK;
+}
+
+// How many consecutive flag values one rank-group launch of this shape consumes,
+// so that a caller who hands out sequence numbers by value (testTransmit's `step`)
+// knows how far apart they must lie.
+extern "C" int vr_rank_flags_used(vr_ctx *ctx, int algo, size_t nelems, uint32_t groups,
+                                  uint32_t subgroups, uint32_t *flags_used) {
+  if (!ctx || !flags_used) return fail(VR_ERR_INVALID, "null argument");
+  if (int rc = use_device(ctx)) return rc;
+  const AlgoInfo *a = algo_info(algo);
+  if (!a) return fail(VR_ERR_ALGO, "unknown algo");
+  const int N = ctx->nranks;
+  const void *table[VR_MAX_RANKS];
+  for (int r = 0; r < N; ++r) table[r] = nullptr;          // address 0: aligned to everything
+  size_t work = 0;
+  if (a->allgather) {
+    work = nelems * 2;
+    if (work % (size_t)a->msg_bytes) return fail(VR_ERR_UNEVEN, "nelems " + std::to_string(nelems));
+  } else if (nelems == 0) {
+    *flags_used = 0;
+    return VR_OK;
+  } else {
+    const size_t msgs = nelems * 2 / (size_t)a->msg_bytes;
+    if (msgs * (size_t)a->msg_bytes != nelems * 2 || msgs % (size_t)N) return fail(VR_ERR_UNEVEN, "nelems " + std::to_string(nelems));
+    work = nelems * 2 / (size_t)N;
+  }
+  const int vec_halves = a->msg_bytes == 16 || (format_widens_with_alignment(ctx, a) && (work / 2) % 8 == 0) ? 8 : 4;
+  WireSinks k;
+  const uint32_t wpr_max = wire_wpr_max(ctx);
+  k.layout = wl::layout_for(N, wpr_max, true);
+  k.wpr_max = wpr_max;
+  k.simple_ok = true;
+  const uint64_t wires = (uint64_t)groups * subgroups;
+  WirePlan plan;
+  if (int rc = plan_wire(ctx, a, work, vec_halves, wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires, k, &plan))
+    return rc;
+  *flags_used = plan.flags_used;
   return VR_OK;
 }
 
@@ -368,8 +564,9 @@ extern "C" int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, 
                                  void *output, void *scatter_buf, void *gather_buf,
                                  void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
                                  size_t nelems, uint32_t *seq_no) {
-  return allreduce_rank(ctx, stream, algo, rank, input, output, scatter_buf, gather_buf, peer_buf0,
-                        peer_buf1, sink_bytes, nelems, seq_no, 0);
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  if (int rc = one_rank_tables(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, p0, p1)) return rc;
+  return allreduce_ranks(ctx, stream, algo, rank, 1, &input, &output, p0, p1, sink_bytes, nelems, seq_no, 0);
 }
 
 // testTransmit's per-rank form with a user grid (main.cpp:67-71, 289-294): every
@@ -379,57 +576,102 @@ extern "C" int vr_allreduce_rank_grid(vr_ctx *ctx, void *stream, int algo, int r
                                       void *const peer_buf0[], void *const peer_buf1[],
                                       size_t sink_bytes, size_t nelems, uint32_t seq_no,
                                       uint32_t groups, uint32_t subgroups, uint32_t simd) {
-  if (subgroups % 4 != 0) return fail(VR_ERR_GEOMETRY, "subgroups = " + std::to_string(subgroups));
-  if (simd != 16 && simd != 32) return fail(VR_ERR_SUBGROUP, "simd = " + std::to_string(simd));
-  if (groups == 0 || subgroups == 0) return fail(VR_ERR_INVALID, "empty grid");
-  const uint64_t wires = (uint64_t)groups * subgroups;
+  uint32_t wires = 0;
+  if (int rc = check_grid(groups, subgroups, simd, &wires)) return rc;
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  if (int rc = one_rank_tables(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, p0, p1)) return rc;
   uint32_t seq = seq_no;
-  return allreduce_rank(ctx, stream, algo, rank, input, output, scatter_buf, gather_buf, peer_buf0,
-                        peer_buf1, sink_bytes, nelems, &seq,
-                        wires > 0xffffffffull ? 0xffffffffu : (uint32_t)wires);
+  return allreduce_ranks(ctx, stream, algo, rank, 1, &input, &output, p0, p1, sink_bytes, nelems, &seq, wires);
 }
 
-// One rank of the ring all-gather (AllGather(input, output, nelems, rank, seqNo, scatterBuf,
-// gatherBuf, peerBuf0, peerBuf1), allgather.hpp:19-29, 58-70).
-extern "C" int vr_allgather_rank(vr_ctx *ctx, void *stream, int algo, int rank, const void *input,
-                                 void *output, void *scatter_buf, void *gather_buf,
-                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
-                                 size_t nelems, uint32_t *seq_no) {
+extern "C" int vr_allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first_rank, int nranks_here,
+                                  void *const inputs[], void *const outputs[], void *const peer_buf0[],
+                                  void *const peer_buf1[], size_t sink_bytes, size_t nelems,
+                                  uint32_t *seq_no) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  return allreduce_ranks(ctx, stream, algo, first_rank, nranks_here, inputs, outputs, peer_buf0, peer_buf1,
+                         sink_bytes, nelems, seq_no, 0);
+}
+
+// Ranks [first, first + count) of the ring all-gather (AllGather(input, output, nelems,
+// rank, seqNo, scatterBuf, gatherBuf, peerBuf0, peerBuf1), allgather.hpp:19-29, 58-70).
+static int allgather_ranks(vr_ctx *ctx, void *stream, int algo, int first, int count,
+                           const void *const inputs[], void *const outputs[], void *const peer_buf0[],
+                           void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no,
+                           uint32_t user_wires) {
   if (int rc = use_device(ctx)) return rc;
   const AlgoInfo *a = algo_info(algo);
   if (!a || !a->allgather) return fail(VR_ERR_ALGO, "not an all-gather algo");
   const int N = ctx->nranks;
-  if (rank < 0 || rank >= N) return fail(VR_ERR_INVALID, "rank out of range");
-  if (!seq_no) return fail(VR_ERR_INVALID, "a one-rank launch needs the caller's sequence number");
-  // allgather.hpp:104-117 for this rank's pointers
-  const void *ins[VR_MAX_RANKS];
-  void *outs[VR_MAX_RANKS];
-  for (int r = 0; r < N; ++r) {
-    ins[r] = input;
-    outs[r] = output;
-  }
-  if (int rc = vr_check_allgather(algo, N, ins, outs, nelems, nullptr)) return rc;
+  if (first < 0 || count < 1 || first + count > N) return fail(VR_ERR_INVALID, "rank out of range");
+  if (!inputs || !outputs) return fail(VR_ERR_INVALID, "null buffer table");
+  if (!seq_no) return fail(VR_ERR_INVALID, "a rank-group launch needs the caller's sequence number");
   const size_t bytes = nelems * 2;
-  const char *own_slot = static_cast<const char *>(output) + (size_t)rank * bytes;
-  const uintptr_t x = (uintptr_t)input, y = (uintptr_t)output;
-  if (x < y + bytes * N && y < x + bytes && (const void *)own_slot != input)
-    return fail(VR_ERR_OVERLAP, "input overlaps output other than as its own slot");
-  WireSinks k;
-  if (int rc = rank_sinks(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
   PtrTable in, out;
   memset(&in, 0, sizeof in);
   memset(&out, 0, sizeof out);
-  in.p[rank] = const_cast<void *>(input);
-  out.p[rank] = output;
+  for (int i = 0; i < count; ++i) {
+    const int rank = first + i;
+    // allgather.hpp:104-117 for one rank's pointers at a time
+    const void *ins[VR_MAX_RANKS];
+    void *outs[VR_MAX_RANKS];
+    for (int r = 0; r < N; ++r) {
+      ins[r] = inputs[i];
+      outs[r] = outputs[i];
+    }
+    if (int rc = vr_check_allgather(algo, N, ins, outs, nelems, nullptr)) return rc;
+    const char *own_slot = static_cast<const char *>(outputs[i]) + (size_t)rank * bytes;
+    const uintptr_t x = (uintptr_t)inputs[i], y = (uintptr_t)outputs[i];
+    if (x < y + bytes * N && y < x + bytes && (const void *)own_slot != inputs[i])
+      return fail(VR_ERR_OVERLAP, "input overlaps output other than as its own slot");
+    in.p[rank] = const_cast<void *>(inputs[i]);
+    out.p[rank] = outputs[i];
+  }
+  WireSinks k;
+  if (int rc = group_sinks(ctx, peer_buf0, peer_buf1, sink_bytes, &k)) return rc;
   vr_geometry geom;
   if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
-  const WireLaunch wlch = {&k, nullptr, ctx->status, rank, false};
+  if (int rc = admit_group_launch(ctx, k.scatter[0], stream, first, count, *seq_no)) return rc;
+  const WireLaunch wlch = {&k, nullptr, ctx->status, first, count, false};
   uint32_t seq = *seq_no, used = 0;
   // messages are 16 bytes, so every pointer and the slice allow 16-byte accesses
-  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, bytes, 8, &seq, 0, &used, wlch)) return rc;
+  if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, bytes, 8, &seq, user_wires, &used, wlch))
+    return rc;
   *seq_no = seq + (used > geom.steps ? used : geom.steps);
   if (*seq_no == 0) *seq_no = 1;
   return VR_OK;
+}
+
+extern "C" int vr_allgather_rank(vr_ctx *ctx, void *stream, int algo, int rank, const void *input,
+                                 void *output, void *scatter_buf, void *gather_buf,
+                                 void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
+                                 size_t nelems, uint32_t *seq_no) {
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  if (int rc = one_rank_tables(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, p0, p1)) return rc;
+  return allgather_ranks(ctx, stream, algo, rank, 1, &input, &output, p0, p1, sink_bytes, nelems, seq_no, 0);
+}
+
+// testAllgather's per-rank form with a user grid (allreduce.cpp:1191-1213, main.cpp:110-166).
+extern "C" int vr_allgather_rank_grid(vr_ctx *ctx, void *stream, int algo, int rank, const void *input,
+                                      void *output, void *scatter_buf, void *gather_buf,
+                                      void *const peer_buf0[], void *const peer_buf1[],
+                                      size_t sink_bytes, size_t nelems, uint32_t seq_no,
+                                      uint32_t groups, uint32_t subgroups, uint32_t simd) {
+  uint32_t wires = 0;
+  if (int rc = check_grid(groups, subgroups, simd, &wires)) return rc;
+  void *p0[VR_MAX_RANKS] = {}, *p1[VR_MAX_RANKS] = {};
+  if (int rc = one_rank_tables(ctx, rank, scatter_buf, gather_buf, peer_buf0, peer_buf1, p0, p1)) return rc;
+  uint32_t seq = seq_no;
+  return allgather_ranks(ctx, stream, algo, rank, 1, &input, &output, p0, p1, sink_bytes, nelems, &seq, wires);
+}
+
+extern "C" int vr_allgather_ranks(vr_ctx *ctx, void *stream, int algo, int first_rank, int nranks_here,
+                                  const void *const inputs[], void *const outputs[],
+                                  void *const peer_buf0[], void *const peer_buf1[], size_t sink_bytes,
+                                  size_t nelems, uint32_t *seq_no) {
+  if (!ctx) return fail(VR_ERR_INVALID, "null ctx");
+  return allgather_ranks(ctx, stream, algo, first_rank, nranks_here, inputs, outputs, peer_buf0, peer_buf1,
+                         sink_bytes, nelems, seq_no, 0);
 }
 
 // Reads one time-out word; if set, resets it and reports the time-out.
@@ -449,20 +691,18 @@ extern "C" int vr_ctx_check(vr_ctx *ctx, void *stream) {
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
   bool timed_out = false;
   if (int rc = check_status_word(ctx->status, &timed_out)) return rc;
-  if (timed_out && ctx->wire.ready) {
-    // A poll gave up: results of that launch are undefined and half-delivered
-    // messages may still sit in the sinks.  Start over from clean scratch.
+  if (!timed_out) return VR_OK;
+  // A poll gave up: results of that launch are undefined and half-delivered
+  // messages may still sit in the sinks.  Scratch the context owns starts over
+  // from zeros; vr_allreduce_static clears what it uses in every call anyway; sinks
+  // a caller handed to vr_allreduce_rank* / vr_allreduce_ranks are the caller's to
+  // zero again.
+  if (ctx->wire.ready) {
     if (int rc = wire_clear(ctx->wire.sinks, ctx->nranks, (hipStream_t)stream)) return rc;
     ctx->wire.hist.used = false;
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
   }
-  if (ctx->static_used) {
-    WireSinks k;
-    uint32_t *word = nullptr;
-    if (int rc = static_sinks(ctx, &k, &word)) return rc;
-    if (int rc = check_status_word(word, &timed_out)) return rc;   // its sinks are cleared by every call
-  }
-  if (timed_out)
-    return fail(VR_ERR_TIMEOUT, "a wire-transport poll exceeded the spin limit; scratch was reset");
-  return VR_OK;
+  return fail(VR_ERR_TIMEOUT, std::string("a wire-transport poll exceeded the spin limit; ") +
+                                  (ctx->wire.ready ? "the context's own scratch was reset; " : "") +
+                                  "caller-owned sinks of rank-group launches must be zeroed again by their owner");
 }

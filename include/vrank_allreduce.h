@@ -27,6 +27,13 @@
  *                        ParallelTransmit / BisectPTransmit ctors    parallel_transmit.hpp:36-60,
  *                                                                    bisect_transmit.hpp:427-482
  *   vr_allgather_rank <- AllGather(input, output, nelems, rank, seqNo, ...)  allgather.hpp:19-29, 58-70
+ *   vr_allgather_grid, vr_allgather_rank_grid
+ *                     <- testAllgather<T>(algo, nd_range, input, output, ipcbuf0, ipcbuf1, peerbuf0,
+ *                        peerbuf1, nelems, rank, world, step, subgroup, queue)  allreduce.cpp:1191-1213,
+ *                        called by benchAllgather with the -g/-w/-s grid    main.cpp:110-166, 296-314
+ *   vr_allreduce_ranks, vr_allgather_ranks
+ *                     <- the same constructors for a process that holds k of the N ranks
+ *                        (the reference always holds one: main.cpp:212-227)
  *   vr_rank_scratch_bytes <- interm_size = world * 8 MiB             main.cpp:241
  *   vr_ipc_open_all   <- open_all_ipc_mems                           ipc_exchange.cpp:277-311
  *                        (un_allgather over AF_UNIX sockets,         ipc_exchange.cpp:173-265)
@@ -179,12 +186,22 @@ int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void 
  *              16-byte aligned, and was zeroed once before the first launch.
  *   seq_no   : in/out; must be the same on every rank and only ever grow; a
  *              change of algo needs freshly zeroed sinks.
- * Same validation and error codes as vr_allreduce for this rank's pointers; in
- * addition, when nelems / nranks is a multiple of 8 elements the chunk travels
- * with 16-byte accesses on every rank, and input and output must be 16-byte
- * aligned (VR_ERR_UNALIGNED otherwise).  The
- * library neither allocates nor clears anything here.  vr_ctx_check(ctx, stream)
- * reports a time-out of this context's launches. */
+ * Same validation and error codes as vr_allreduce for this rank's pointers
+ * (calcWorkSize: alignment to the protocol's message_t).  Only `parallel`, and
+ * the Rt64_128 families when "wire_fenced" selects a flag-word format, move 16
+ * bytes per lane whenever nelems / nranks is a multiple of 8 elements, on every
+ * rank alike; input and output must then be 16-byte aligned (VR_ERR_UNALIGNED).
+ * The library neither allocates nor clears anything here.  vr_ctx_check(ctx,
+ * stream) reports a time-out of this context's launches; after one, the caller
+ * zeroes its sinks again.
+ * Concurrency inside one process: every launch of a collective needs a stream of
+ * its own and a hardware queue of its own.  A process has GPU_MAX_HW_QUEUES of
+ * them (4 unless the environment says otherwise), so at most that many one-rank
+ * launches can form a collective in one process; a launch that would exceed it,
+ * or that shares a stream with another rank of the same collective (same sinks,
+ * same seq_no), is refused with VR_ERR_INVALID before anything is enqueued.
+ * Hold several ranks per launch (vr_allreduce_ranks) or run the ranks in
+ * separate processes instead. */
 int vr_allreduce_rank(vr_ctx *ctx, void *stream, int algo, int rank, void *input, void *output,
                       void *scatter_buf, void *gather_buf, void *const peer_buf0[],
                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
@@ -202,6 +219,33 @@ int vr_allreduce_rank_grid(vr_ctx *ctx, void *stream, int algo, int rank, void *
 int vr_allgather_rank(vr_ctx *ctx, void *stream, int algo, int rank, const void *input, void *output,
                       void *scatter_buf, void *gather_buf, void *const peer_buf0[],
                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+/* The same with the test harness's user grid: testAllgather<T>(algo, nd_range, input,
+ * output, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1, nelems, rank, world, step, subgroup,
+ * queue) (allreduce.cpp:1191-1213; benchAllgather, main.cpp:110-166).  Rejections as
+ * vr_allreduce_grid. */
+int vr_allgather_rank_grid(vr_ctx *ctx, void *stream, int algo, int rank, const void *input,
+                           void *output, void *scatter_buf, void *gather_buf, void *const peer_buf0[],
+                           void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t seq_no,
+                           uint32_t groups, uint32_t subgroups, uint32_t simd);
+/* Ranks [first_rank, first_rank + nranks_here) of a collective in ONE launch: what a
+ * process that owns k of the N ranks enqueues (the reference's processes own one
+ * each, allreduce.hpp:18-28).  inputs[i] / outputs[i] belong to rank first_rank + i
+ * (outputs NULL, or an entry NULL = in place); peer_buf0[] / peer_buf1[] hold every
+ * rank's scatter / gather sink, the launch's own ranks included.  Otherwise the
+ * contract of vr_allreduce_rank / vr_allgather_rank.  N ranks on a process's 4
+ * hardware queues: N / 4 ranks per launch on 4 streams. */
+int vr_allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first_rank, int nranks_here,
+                       void *const inputs[], void *const outputs[], void *const peer_buf0[],
+                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+int vr_allgather_ranks(vr_ctx *ctx, void *stream, int algo, int first_rank, int nranks_here,
+                       const void *const inputs[], void *const outputs[], void *const peer_buf0[],
+                       void *const peer_buf1[], size_t sink_bytes, size_t nelems, uint32_t *seq_no);
+/* Consecutive flag values one rank-group launch of this shape consumes (groups = 0:
+ * the library's own grid).  Sequence numbers of successive launches on the same
+ * sinks must lie at least this far apart; main.cpp's fixed offsets (flag, +100,
+ * +150, +200; l.67-106) allow 50. */
+int vr_rank_flags_used(vr_ctx *ctx, int algo, size_t nelems, uint32_t groups, uint32_t subgroups,
+                       uint32_t *flags_used);
 /* Bytes a scatter sink (and equally a gather sink) must hold for this context's
  * rank count, device and "wire_blocks_per_cu" setting. */
 int vr_rank_scratch_bytes(const vr_ctx *ctx, size_t *sink_bytes);
@@ -233,9 +277,10 @@ int vr_ipc_barrier(int rank, int world, const char *instance, int generation);
  * Limits: at most 8 ranks, at most 256 MiB (134217728 elements) per rank, every
  * all-reduce algo except simple_transmit; 32 wires per rank.  Beyond them:
  * VR_ERR_INVALID.  Every context on a GPU shares that GPU's region and each call
- * clears it first (on `stream`), so calls that overlap in time on one GPU race:
- * keep them on one stream or otherwise ordered.  Time-outs are reported by
- * vr_ctx_check like those of vr_allreduce. */
+ * first clears the message slots it is about to use (a fill kernel on `stream`),
+ * so calls that overlap in time on one GPU race: keep them on one stream or
+ * otherwise ordered.  A time-out is recorded in the calling context's own status
+ * word and reported by vr_ctx_check like those of vr_allreduce. */
 int vr_allreduce_static(vr_ctx *ctx, void *stream, int algo, void *const bufs[], void *const outs[],
                         size_t nelems);
 
@@ -247,8 +292,17 @@ int vr_allreduce_grid(vr_ctx *ctx, void *stream, int algo, int transport, void *
                       void *const outs[], size_t nelems, uint32_t seq_no, uint32_t groups,
                       uint32_t subgroups, uint32_t simd);
 
+/* testAllgather with a user grid for all ranks at once (allreduce.cpp:1191-1213,
+ * main.cpp:110-166, 293-307): `groups` x `subgroups` sub-groups of `simd` lanes per
+ * rank; same rejections as vr_allreduce_grid. */
+int vr_allgather_grid(vr_ctx *ctx, void *stream, int algo, int transport, const void *const inputs[],
+                      void *const outputs[], size_t nelems, uint32_t seq_no, uint32_t groups,
+                      uint32_t subgroups, uint32_t simd);
+
 /* After a wire-transport launch has completed: VR_OK, or VR_ERR_TIMEOUT if any
- * poll gave up.  (Synchronises `stream`.) */
+ * poll gave up.  (Synchronises `stream`.)  After a time-out the context's own
+ * scratch has been zeroed again; sinks a caller handed to the rank-group launches
+ * are the caller's to zero. */
 int vr_ctx_check(vr_ctx *ctx, void *stream);
 /* Poll budget of the wire transport's bounded spin (0 = library default). */
 int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
@@ -262,10 +316,12 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch
  * covers; chunks longer than this, at most 1 GiB, take several launches);
- * for the wire transport "wire_fenced" (the Rt64_128 families: 1 = payload lines
- * with a separate flag word ordered by agent-scope release/acquire fences, 2 =
- * self-validating 8-byte messages, instead of the reference's 128 / 256-byte
- * messages with a flag in every 64 bytes) and
+ * for the wire transport "wire_fenced" (the Rt64_128 families, instead of the
+ * reference's 128 / 256-byte messages with a flag in every 64 bytes: 1 = payload
+ * lines with a separate flag word ordered by agent-scope release/acquire fences,
+ * 2 = self-validating 8-byte messages, 3 = as 1 with the payload stored written
+ * through at agent scope, 4 = flag words with every access at agent scope, ordered
+ * by store completion alone, no cache maintenance) and
  * "wire_cooperative" (1 = cooperative launch; by default a plain launch: the
  * library sizes every grid within the occupancy query's bound, so it is
  * co-resident on an otherwise idle device),
@@ -287,6 +343,13 @@ int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);
  * times in milliseconds (ms_out[iters]).  Out-of-place when outs != NULL. */
 int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
                       void *const outs[], size_t nelems, int iters, float *ms_out);
+/* `groups` event pairs, each around `per_group` back-to-back vr_allreduce calls made
+ * exactly as a caller makes them.  ms_out[g] = device time of group g / per_group;
+ * *host_call_us (optional) = host wall time one vr_allreduce call takes to return
+ * (validation, launch heuristics, kernel enqueue), averaged over all calls. */
+int vr_time_allreduce_grouped(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                              void *const outs[], size_t nelems, int groups, int per_group,
+                              float *ms_out, double *host_call_us);
 int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transport,
                       const void *const inputs[], void *const outputs[], size_t nelems, int iters,
                       float *ms_out);

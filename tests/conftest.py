@@ -18,7 +18,8 @@ def pytest_configure(config):
              os.path.join(ROOT, "oracle", "libvr_oracle.so"),
              os.path.join(ROOT, "tests", "cpp", "test_host_api"),
              os.path.join(ROOT, "tests", "cpp", "test_graph"),
-             os.path.join(ROOT, "tests", "cpp", "test_wire_layout")]
+             os.path.join(ROOT, "tests", "cpp", "test_wire_layout"),
+             os.path.join(ROOT, "tests", "cpp", "test_verify")]
     if not all(os.path.exists(p) for p in built):
         import __graft_entry__
         __graft_entry__.build()

@@ -146,6 +146,66 @@ static int run_all() {
       EXPECT(b.mismatches(want) == 0);
     }
   }
+  // --- testAllgather with a user grid, both transports, then the reference's host checks --------------
+  {
+    VirtualRanks ranks(4);
+    ranks.reserveWire();
+    for (int transport : {VR_TRANSPORT_DIRECT, VR_TRANSPORT_WIRE}) {
+      ranks.setTransport(transport);
+      uint32_t step = 0xe00f100f;
+      for (const char *algo : {"allgather_small", "allgather_simple"}) {
+        for (LaunchParam grid : {LaunchParam{1, 4, 16}, LaunchParam{7, 8, 16}, LaunchParam{19, 32, 32}}) {
+          Ranks in(4, 8 * 1237, 53), out(4, 8 * 1237, 54, 4);
+          std::vector<uint16_t> want(4 * in.nelems);
+          auto hp = in.host_ptrs();
+          vro_allgather(want.data(), hp.data(), 4, in.nelems);
+          testAllgather<half_bits>(algo, grid, ranks, in.dev.data(), out.dev.data(), in.nelems, step);
+          ranks.wait();
+          step += 100;
+          EXPECT(out.mismatches(want) == 0);
+        }
+      }
+    }
+    ranks.setTransport(VR_TRANSPORT_DEFAULT);
+    EXPECT(thrown([&] { Ranks in(4, 64, 1), out(4, 64, 2, 4);
+                        testAllgather<half_bits>("small", {1, 4, 16}, ranks, in.dev.data(), out.dev.data(), in.nelems, 1); }) ==
+           "Transmit type not support");
+    EXPECT(thrown([&] { Ranks in(4, 64, 1), out(4, 64, 2, 4);
+                        testAllgather<half_bits>("allgather_small", {1, 2, 16}, ranks, in.dev.data(), out.dev.data(), in.nelems, 1); }) ==
+           "Subgroup numbers must be multiple of 4");
+  }
+  // --- verifyTransmit / verifyAllgather on what the device produced from fill_pattern (main.cpp -v) ----
+  {
+    const int W = 8;
+    const size_t n = 14336;
+    VirtualRanks ranks(W);
+    std::vector<half_bits *> dev(W), gathered(W);
+    std::vector<uint16_t> host(n);
+    for (int r = 0; r < W; ++r) {
+      void *p;
+      check(vr_malloc(0, n * 2, &p));
+      dev[r] = (half_bits *)p;
+      check(vr_malloc(0, n * 2 * W, &p));
+      gathered[r] = (half_bits *)p;
+      check(vr_memset(p, 1, n * 2 * W));
+      vr_fill_pattern(host.data(), r, n);
+      check(vr_copy_to_device(dev[r], host.data(), n * 2));
+    }
+    testAllgather<half_bits>("allgather_simple", {7, 8, 16}, ranks, dev.data(), gathered.data(), n, 5);
+    ranks.wait();
+    testTransmit<half_bits>("bisect", {13, 8, 16}, ranks, dev.data(), n, 0xe00f100f);
+    ranks.wait();
+    std::vector<half_bits> got(n), cat(n * W);
+    for (int r = 0; r < W; ++r) {
+      size_t bad = 99;
+      check(vr_copy_to_host(got.data(), dev[r], n * 2));
+      EXPECT(verifyTransmit<half_bits>(nullptr, got.data(), 0xe00f100f, r, W, 16, n, &bad) == 0 && bad == 0);
+      check(vr_copy_to_host(cat.data(), gathered[r], n * 2 * W));
+      EXPECT(verifyAllgather<half_bits>(cat.data(), r, W, n, &bad) == 0 && bad == 0);
+      vr_free(dev[r]);
+      vr_free(gathered[r]);
+    }
+  }
   // --- bfloat16 through the same templates -----------------------------------------------------------
   {
     VirtualRanks ranks(8);
@@ -251,6 +311,26 @@ static int run_all() {
       }
       wait_all();
       EXPECT(out.mismatches(want) == 0);
+    }
+    {  // testAllgather<T>(algo, nd_range, input, output, ipcbuf0, ipcbuf1, peerbuf0, peerbuf1, nelems, rank, world, step, subgroup, queue)
+      for (const char *algo : {"allgather_small", "allgather_simple"}) {
+        for (LaunchParam grid : {LaunchParam{1, 4, 16}, LaunchParam{13, 8, 16}}) {
+          zero();
+          Ranks in(W, 8 * 2049, 87), out(W, 8 * 2049, 88, W);
+          std::vector<uint16_t> want(W * in.nelems);
+          auto hp = in.host_ptrs();
+          vro_allgather(want.data(), hp.data(), W, in.nelems);
+          for (int r = 0; r < W; ++r)
+            testAllgather<half_bits>(algo, grid, in.dev[r], out.dev[r], ipcbuf0[r], ipcbuf1[r], ipcbuf0, ipcbuf1,
+                                     in.nelems, r, W, step, 16, streams[r]);
+          wait_all();
+          step += 1000;
+          EXPECT(out.mismatches(want) == 0);
+        }
+      }
+      Ranks in(W, 64, 1), out(W, 64, 2, W);
+      EXPECT(thrown([&] { testAllgather<half_bits>("simple", {1, 4, 16}, in.dev[0], out.dev[0], ipcbuf0[0], ipcbuf1[0], ipcbuf0, ipcbuf1, in.nelems, 0, W, 1, 16); }) ==
+             "Transmit type not support");
     }
     {  // the constructor's exceptions, per rank
       Ranks b(W, W * 64, 86);

@@ -14,6 +14,7 @@ CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
 CPP_TEST = os.path.join(ROOT, "tests", "cpp", "test_host_api")
 GRAPH_TEST = os.path.join(ROOT, "tests", "cpp", "test_graph")
 LAYOUT_TEST = os.path.join(ROOT, "tests", "cpp", "test_wire_layout")
+VERIFY_TEST = os.path.join(ROOT, "tests", "cpp", "test_verify")
 
 
 def run(cmd, **kw):
@@ -32,10 +33,19 @@ def test_wire_sinks_hold_every_slot_the_kernels_index():
     assert r.returncode == 0 and " 0 failures" in r.stdout, r.stdout
 
 
+def test_host_side_checks_of_the_cpp_header():
+    """vrank::verifyTransmit / verifyAllReduce / verifyAllgather (allreduce.cpp:519-585,
+    832-838) and the element arithmetic under them, against the oracle; CPU only."""
+    r = run([VERIFY_TEST], timeout=120)
+    assert r.returncode == 0 and "verify ok" in r.stdout, r.stdout[-2000:]
+
+
 def test_cli_rejects_bad_arguments_like_the_reference():
     r = run([CLI, "-n", "1K", "-a", "tree"])
     assert r.returncode == 1 and "Transmit type not support" in r.stdout
     r = run([CLI, "-n", "1K", "-a", "small", "-g", "4", "-w", "2"])
+    assert r.returncode == 1 and "Subgroup numbers must be multiple of 4" in r.stdout
+    r = run([CLI, "-n", "1K", "-a", "allgather_small", "-g", "4", "-w", "6"])     # all-gather takes the grid too
     assert r.returncode == 1 and "Subgroup numbers must be multiple of 4" in r.stdout
     r = run([CLI, "--help"])
     assert r.returncode == 0 and "usage" in r.stdout
@@ -114,6 +124,19 @@ def test_cli_verify_sweep(world, algo):
                     timeout=60)
             assert r.returncode == 0, r.stdout
             assert "Error Compare" not in r.stdout and "match" in r.stdout, (n, g, w, r.stdout[-400:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transport", ["direct", "wire"])
+def test_cli_allgather_honours_the_grid(transport):
+    """-s is passed on for all-gather algos as for all-reduce ones: a sub-group size the
+    dispatcher does not instantiate is rejected (allreduce.cpp:917), 16 and 32 run."""
+    base = [CLI, "-v", "-n", "2048", "-r", "4", "-a", "allgather_simple", "-t", transport, "-g", "7", "-w", "8"]
+    r = run(base + ["-s", "8"], timeout=60)
+    assert r.returncode == 1 and "Unsupported Sub-group size" in r.stdout, r.stdout
+    for simd in ("16", "32"):
+        r = run(base + ["-s", simd], timeout=60)
+        assert r.returncode == 0 and "gathered elements match" in r.stdout, r.stdout
 
 
 @pytest.mark.gpu

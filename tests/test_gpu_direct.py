@@ -349,6 +349,47 @@ def test_allgather(ctxs, oracle, nranks, algo):
                 assert (got[r] == want).all(), (n, r, alias)
 
 
+@pytest.mark.parametrize("transport", ["direct", "wire"])
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_allgather_result_independent_of_grid(ctxs, oracle, algo, transport):
+    """testAllgather takes the harness's -g / -w / -s grid (allreduce.cpp:1191-1213,
+    main.cpp:293-307): the gathered bytes never depend on it, and the grids
+    main.cpp or the dispatcher reject are rejected here."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    tr = vr.TRANSPORT_WIRE if transport == "wire" else vr.TRANSPORT_DIRECT
+    ctx = ctxs[4]
+    n = 14336
+    ins = H.make_inputs(oracle, 4, n, 7300, DIST_UNIFORM, -2.0, 2.0)
+    want = oracle.allgather(ins)
+    srcs = [DeviceBuffer(n * 2) for _ in range(4)]
+    outs = [DeviceBuffer(4 * n * 2) for _ in range(4)]
+    for s, a in zip(srcs, ins):
+        s.upload(a)
+    seq = 0xE00F100F
+    for groups in (1, 2, 7, 13, 19, 64):
+        for subgroups in (4, 8, 32, 64):
+            for o in outs:
+                o.fill(0x01)
+            ctx.allgather_grid(algo, [s.ptr for s in srcs], [o.ptr for o in outs], n, groups, subgroups,
+                               simd=32 if groups == 7 else 16, transport=tr, seq_no=seq)
+            ctx.check()
+            seq += 100
+            for r in range(4):
+                assert (outs[r].download(np.uint16, 4 * n) == want).all(), (algo, transport, groups, subgroups, r)
+    for bad_w, code in ((2, "GEOMETRY"), (6, "GEOMETRY")):
+        with pytest.raises(vr.VRError) as e:
+            ctx.allgather_grid(algo, [s.ptr for s in srcs], [o.ptr for o in outs], n, 4, bad_w, transport=tr)
+        assert e.value.code == code
+    with pytest.raises(vr.VRError) as e:
+        ctx.allgather_grid(algo, [s.ptr for s in srcs], [o.ptr for o in outs], n, 4, 4, simd=8, transport=tr)
+    assert e.value.code == "SUBGROUP"
+    with pytest.raises(vr.VRError) as e:
+        ctx.allgather_grid("simple", [s.ptr for s in srcs], [o.ptr for o in outs], n, 4, 4, transport=tr)
+    assert e.value.code == "ALGO"
+    for b in srcs + outs:
+        b.free()
+
+
 def test_config4_allgather_8mib(ctxs, oracle):
     ins = H.make_inputs(oracle, 4, 4194304, 4000, DIST_UNIFORM, -2.0, 2.0)
     want = oracle.allgather(ins)

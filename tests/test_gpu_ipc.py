@@ -17,13 +17,15 @@ CLI = os.path.join(ROOT, "gpu_ipc_example_amd", "vr_main")
 _runs = [0]
 
 
-def run_ranks(world, extra, per_rank=None, timeout=100):
-    """Start `world` rank processes, wait for all; returns [(returncode, output)]."""
+def run_ranks(world, extra, per_rank=None, timeout=100, ranks_here=1):
+    """Start one process per `ranks_here` ranks, wait for all; returns [(returncode, output)]."""
     _runs[0] += 1
     instance = "g%d_%d" % (os.getpid(), _runs[0])
     procs = []
-    for r in range(world):
+    for r in range(0, world, ranks_here):
         cmd = [CLI, "-r", str(world), "--rank", str(r), "-i", instance] + extra + (per_rank(r) if per_rank else [])
+        if ranks_here > 1:
+            cmd += ["--ranks-here", str(ranks_here)]
         procs.append(subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
     out = []
     for p in procs:
@@ -64,6 +66,61 @@ def test_seeded_inputs_match_the_oracle_across_processes(oracle, tmp_path, world
     for r in range(world):
         got = np.fromfile(tmp_path / ("out%d.bin" % r), np.uint16)
         assert len(got) == n and oracle.count_mismatch(got, want) == 0, (algo, r)
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_allgather_across_processes(oracle, tmp_path, world, algo):
+    """benchAllgather per process (main.cpp:110-166, 296-314): output memset to 1, -v
+    through verifyAllgather; with and without the -g / -w grid; then seeded inputs
+    whose dumped outputs are compared with the oracle's all-gather."""
+    for grid in ([], ["-g", "7", "-w", "8"], ["-g", "19", "-w", "32", "-s", "32"]):
+        for n in (16384, 14336 * 4):
+            res = run_ranks(world, ["-v", "-n", str(n), "-a", algo] + grid)
+            for r, (rc, text) in enumerate(res):
+                assert rc == 0, (algo, n, grid, r, text)
+                assert "gathered elements match" in text and "Error Compare" not in text, (algo, n, grid, r, text)
+    n = 1 << 18
+    seed = 9300 + world
+    res = run_ranks(world, ["-n", str(n), "-a", algo, "--seed", str(seed), "-g", "13", "-w", "8"],
+                    per_rank=lambda r: ["--dump", str(tmp_path / ("ag%d.bin" % r))])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0, (algo, r, text)
+    want = oracle.allgather(H.make_inputs(oracle, world, n, seed))
+    for r in range(world):
+        got = np.fromfile(tmp_path / ("ag%d.bin" % r), np.uint16)
+        assert len(got) == world * n and (got == want).all(), (algo, r)
+
+
+def test_allgather_timed_run_across_processes():
+    res = run_ranks(4, ["-n", "1M", "-a", "allgather_simple", "-g", "16", "-w", "16"])
+    for r, (rc, text) in enumerate(res):
+        assert rc == 0 and "[%d] Running time: " % r in text, (r, text)
+
+
+@pytest.mark.parametrize("world,here,algo", [(8, 4, "parallel"), (8, 4, "bisect"), (8, 2, "simple"),
+                                             (8, 4, "small_ring"), (4, 2, "simple_pcie"),
+                                             (8, 4, "allgather_simple")])
+def test_several_ranks_per_process(oracle, tmp_path, world, here, algo):
+    """world / here processes, each holding `here` ranks in one launch
+    (vr_allreduce_ranks / vr_allgather_ranks) against sinks mapped over IPC."""
+    gather = algo.startswith("allgather")
+    res = run_ranks(world, ["-v", "-n", "16384", "-a", algo], ranks_here=here)
+    for p, (rc, text) in enumerate(res):
+        assert rc == 0 and "Error Compare" not in text, (algo, p, text)
+        for r in range(p * here, (p + 1) * here):
+            assert "[%d] verify: " % r in text and "mismatches" not in text, (algo, r, text)
+    n = 1 << 20
+    seed = 9400 + world + here
+    res = run_ranks(world, ["-n", str(n), "-a", algo, "--seed", str(seed)], ranks_here=here,
+                    per_rank=lambda r: ["--dump", str(tmp_path / "grp.bin")])
+    for p, (rc, text) in enumerate(res):
+        assert rc == 0, (algo, p, text)
+    ins = H.make_inputs(oracle, world, n, seed)
+    want = oracle.allgather(ins) if gather else H.expected(oracle, algo, ins)
+    for r in range(world):
+        got = np.fromfile(str(tmp_path / "grp.bin") + ".%d" % r, np.uint16)
+        assert len(got) == len(want) and oracle.count_mismatch(got, want) == 0, (algo, r)
 
 
 def test_timed_run_protocol_across_processes():

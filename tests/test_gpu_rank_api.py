@@ -213,11 +213,203 @@ def test_rank_call_validates_like_the_constructor(ranks):
     with pytest.raises(vr.VRError) as e:
         c.allreduce_rank("simple", 0, buf.ptr, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 0)
     assert e.value.code == "INVALID"
-    # a chunk of 16-byte multiples travels with 16-byte accesses on every rank
+    # `parallel` (256-byte messages) moves a chunk of 16-byte multiples with 16-byte
+    # accesses on every rank; the 8-byte-message protocols accept what calcWorkSize
+    # accepts (allreduce.hpp:110: alignment to message_t), see the next test
     with pytest.raises(vr.VRError) as e:
-        c.allreduce_rank("simple", 0, buf.ptr + 8, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 1)
+        c.allreduce_rank("parallel", 0, buf.ptr + 8, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 1)
     assert e.value.code == "UNALIGNED" and "16-byte" in e.value.detail
     buf.free()
+
+
+@pytest.mark.parametrize("algo", ["simple", "bisect", "small", "simple_transmit"])
+def test_eight_byte_aligned_buffers_with_sixteen_byte_chunks(ranks, oracle, algo):
+    """message_t of small / simple / bisect is 8 bytes (rt64.hpp:335, rt64_128.hpp:539):
+    an 8-byte-aligned buffer is accepted whatever the chunk length, as by the
+    reference's per-rank calcWorkSize."""
+    R = ranks[4]
+    R.zero()
+    seq = 1
+    for n in (4 * 64, 4 * 8 * 1001):                     # chunks of 16-byte multiples
+        ins = H.make_inputs(oracle, 4, n, 8700 + n)
+        src = H.RankBuffers(4, n, 8)                     # every buffer 8 bytes off a 16-byte boundary
+        src.upload(ins)
+        s0 = [b.ptr for b in R.scatter]
+        s1 = [b.ptr for b in R.gather]
+        nxt = seq
+        for r in range(4):
+            nxt = R.ctx[r].allreduce_rank(algo, r, src.ptrs[r], s0[r], s1[r], s0, s1, R.sink_bytes, n, seq,
+                                          stream=R.handle(r))
+        for r in range(4):
+            R.ctx[r].check(R.handle(r))
+        seq = nxt
+        H.assert_all_ranks_equal(oracle, src.download(), H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+        src.free()
+
+
+class Groups:
+    """N ranks held by N / k launches of k ranks each (vr_allreduce_ranks), one stream
+    per launch: 8 ranks on the 4 hardware queues of one process."""
+
+    def __init__(self, nranks, per_launch):
+        self.n, self.k = nranks, per_launch
+        self.ctx = vr.VirtualRanks(nranks)
+        self.ctx.set_spin_limit(SPIN)
+        self.streams = stream_pool()[:nranks // per_launch]
+        self.sink_bytes = self.ctx.rank_scratch_bytes()
+        self.scatter = [DeviceBuffer(self.sink_bytes) for _ in range(nranks)]
+        self.gather = [DeviceBuffer(self.sink_bytes) for _ in range(nranks)]
+        self.zero()
+
+    def zero(self):
+        for b in self.scatter + self.gather:
+            b.fill(0)
+
+    def handle(self, g):
+        return self.streams[g].handle if self.streams[g] else None
+
+    def check(self):
+        for g in range(len(self.streams)):
+            self.ctx.check(self.handle(g))
+
+    def close(self):
+        for b in self.scatter + self.gather:
+            b.free()
+        self.ctx.close()
+
+
+@pytest.mark.parametrize("nranks,per_launch", [(8, 2), (8, 4), (4, 2)])
+@pytest.mark.parametrize("algo", ["simple", "small", "parallel", "bisect", "simple_ring", "small_pcie"])
+def test_rank_group_launches(oracle, nranks, per_launch, algo):
+    G = Groups(nranks, per_launch)
+    s0 = [b.ptr for b in G.scatter]
+    s1 = [b.ptr for b in G.gather]
+    seq = 1
+    for k, n in enumerate((64 * nranks, 64 * nranks * 33, 1 << 20)):
+        ins = H.make_inputs(oracle, nranks, n, 8800 + 10 * k + nranks)
+        want = H.expected(oracle, algo, ins)
+        for inplace in (True, False):
+            src = H.RankBuffers(nranks, n)
+            src.upload(ins)
+            dst = None
+            if not inplace:
+                dst = H.RankBuffers(nranks, n)
+                dst.fill(0xAB)
+            nxt = seq
+            for g in range(nranks // per_launch):
+                first = g * per_launch
+                nxt = G.ctx.allreduce_ranks(algo, first, src.ptrs[first:first + per_launch], s0, s1, G.sink_bytes,
+                                            n, seq, outs=dst.ptrs[first:first + per_launch] if dst else None,
+                                            stream=G.handle(g))
+            G.check()
+            assert nxt > seq
+            seq = nxt
+            H.assert_all_ranks_equal(oracle, (dst or src).download(), want,
+                                     "%s N=%d k=%d n=%d" % (algo, nranks, per_launch, n))
+            src.free()
+            if dst:
+                dst.free()
+    G.close()
+
+
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_rank_group_allgather(oracle, algo):
+    G = Groups(8, 2)
+    s0 = [b.ptr for b in G.scatter]
+    s1 = [b.ptr for b in G.gather]
+    seq = 1
+    for n in (8, 8 * 1237, 1 << 17):
+        ins = H.make_inputs(oracle, 8, n, 8900 + n)
+        want = oracle.allgather(ins)
+        srcs = [DeviceBuffer(n * 2) for _ in range(8)]
+        outs = [DeviceBuffer(8 * n * 2) for _ in range(8)]
+        for r in range(8):
+            srcs[r].upload(ins[r])
+            outs[r].fill(0x01)
+        nxt = seq
+        for g in range(4):
+            nxt = G.ctx.allgather_ranks(algo, 2 * g, [b.ptr for b in srcs[2 * g:2 * g + 2]],
+                                        [b.ptr for b in outs[2 * g:2 * g + 2]], s0, s1, G.sink_bytes, n, seq,
+                                        stream=G.handle(g))
+        G.check()
+        seq = nxt
+        for r in range(8):
+            assert np.array_equal(outs[r].download(np.uint16, 8 * n), want), (algo, n, r)
+        for b in srcs + outs:
+            b.free()
+    G.close()
+
+
+def test_more_launches_than_hardware_queues_are_refused(oracle):
+    """Eight one-rank launches in one process would need eight hardware queues; a
+    process has four.  The fifth launch of the collective is refused with the
+    remedy instead of ending in a time-out, and so is a second rank on a stream
+    that already carries another rank of the same collective."""
+    R = Groups(8, 1)                                       # sinks for 8 ranks, context, pool of streams
+    R.ctx.set_spin_limit(64)
+    n = 8 * 64
+    src = H.RankBuffers(8, n)
+    src.upload(H.make_inputs(oracle, 8, n, 9000))
+    s0 = [b.ptr for b in R.scatter]
+    s1 = [b.ptr for b in R.gather]
+    pool = stream_pool()
+    handles = [p.handle if p else None for p in pool]
+    for r in range(4):
+        R.ctx.allreduce_rank("simple", r, src.ptrs[r], s0[r], s1[r], s0, s1, R.sink_bytes, n, 7, stream=handles[r])
+    extra = Stream()
+    with pytest.raises(vr.VRError) as e:
+        R.ctx.allreduce_rank("simple", 4, src.ptrs[4], s0[4], s1[4], s0, s1, R.sink_bytes, n, 7, stream=extra.handle)
+    assert e.value.code == "INVALID" and "vr_allreduce_ranks" in e.value.detail
+    with pytest.raises(vr.VRError) as e:
+        R.ctx.allreduce_rank("simple", 5, src.ptrs[5], s0[5], s1[5], s0, s1, R.sink_bytes, n, 7, stream=handles[1])
+    assert e.value.code == "INVALID" and "same stream" in e.value.detail
+    # the four launches that did start give up after 64 polls and drain
+    timed_out = 0
+    for r in range(4):
+        try:
+            R.ctx.check(handles[r])
+        except vr.VRError as err:
+            assert err.code == "TIMEOUT"
+            timed_out += 1
+    assert timed_out >= 1
+    extra.close()
+    src.free()
+    R.close()
+
+
+@pytest.mark.parametrize("algo", ["allgather_small", "allgather_simple"])
+def test_rank_allgather_with_a_user_grid(ranks, oracle, algo):
+    """testAllgather's per-rank form (allreduce.cpp:1191-1213): the -g / -w / -s grid
+    changes the launch, never the gathered bytes."""
+    R = ranks[4]
+    R.zero()
+    s0 = [b.ptr for b in R.scatter]
+    s1 = [b.ptr for b in R.gather]
+    n = 14336
+    ins = H.make_inputs(oracle, 4, n, 9100)
+    want = oracle.allgather(ins)
+    srcs = [DeviceBuffer(n * 2) for _ in range(4)]
+    outs = [DeviceBuffer(4 * n * 2) for _ in range(4)]
+    for r in range(4):
+        srcs[r].upload(ins[r])
+    seq = 0xE00F100F
+    for groups, subgroups, simd in ((1, 4, 16), (7, 8, 16), (19, 32, 32), (64, 64, 16)):
+        for o in outs:
+            o.fill(0x01)
+        for r in range(4):
+            R.ctx[r].allgather_rank_grid(algo, r, srcs[r].ptr, outs[r].ptr, s0[r], s1[r], s0, s1, R.sink_bytes, n,
+                                         seq, groups, subgroups, simd, stream=R.handle(r))
+        for r in range(4):
+            R.ctx[r].check(R.handle(r))
+        seq += 100
+        for r in range(4):
+            assert np.array_equal(outs[r].download(np.uint16, 4 * n), want), (algo, groups, subgroups, r)
+    with pytest.raises(vr.VRError) as e:
+        R.ctx[0].allgather_rank_grid(algo, 0, srcs[0].ptr, outs[0].ptr, s0[0], s1[0], s0, s1, R.sink_bytes, n,
+                                     seq, 4, 2, 16)
+    assert e.value.code == "GEOMETRY"
+    for b in srcs + outs:
+        b.free()
 
 
 @pytest.mark.parametrize("algo", ["simple", "parallel", "small", "bisect"])

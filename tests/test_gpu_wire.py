@@ -239,19 +239,49 @@ def test_allgather_wire(ctxs, oracle, nranks, algo):
                 assert (got[r] == want).all(), (n, r, alias)
 
 
+@pytest.mark.parametrize("fenced", [1, 3, 4])
 @pytest.mark.parametrize("algo", ["simple", "parallel", "bisect", "simple_ring", "simple_pcie",
                                   "simple_pcie_p", "simple_transmit"])
-def test_fenced_flag_word_format(oracle, algo):
-    """The Rt64_128 family can also travel as payload lines + a separate flag word
-    ordered by agent-scope release/acquire fences (no store-atomicity assumption)."""
+def test_fenced_flag_word_format(oracle, algo, fenced):
+    """The Rt64_128 family can also travel as payload lines + a separate flag word:
+    ordered by agent-scope release/acquire fences (1; 3 = payload written through),
+    or by store completion with every access at agent scope (4).  No assumption
+    about store atomicity in any of them."""
     ctx = vr.VirtualRanks(8)
-    ctx.set_tuning(wire_fenced=1)
+    ctx.set_tuning(wire_fenced=fenced)
     for n in (64, 64 * 129, 1 << 18, 32 * 1001):
         if algo in ("simple_ring", "simple_pcie", "simple_pcie_p") and n % 64:
             continue
         ins = H.make_inputs(oracle, 8, n, 6000 + n)
-        got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE)
-        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+        for inplace in (True, False):
+            got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, inplace=inplace)
+            H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+    ctx.close()
+
+
+@pytest.mark.parametrize("fenced", [1, 4])
+@pytest.mark.parametrize("algo", ["parallel", "bisect", "simple_pcie"])
+def test_flag_word_formats_under_repetition(oracle, algo, fenced):
+    """60 launches over the same sinks: slots and flag words are reused with growing
+    flag values, and every tenth result is compared with the oracle."""
+    from gpu_ipc_example_amd.binding import DeviceBuffer
+    ctx = vr.VirtualRanks(8)
+    ctx.set_tuning(wire_fenced=fenced)
+    n = 64 * 1025
+    ins = H.make_inputs(oracle, 8, n, 6900)
+    want = H.expected(oracle, algo, ins)
+    src = [DeviceBuffer(n * 2) for _ in range(8)]
+    dst = [DeviceBuffer(n * 2) for _ in range(8)]
+    for b, a in zip(src, ins):
+        b.upload(a)
+    for it in range(60):
+        ctx.allreduce(algo, [b.ptr for b in src], n, outs=[b.ptr for b in dst], transport=WIRE)
+        if it % 10 == 9:
+            ctx.check()
+            for r, b in enumerate(dst):
+                assert oracle.count_mismatch(b.download(np.uint16, n), want) == 0, (algo, fenced, it, r)
+    for b in src + dst:
+        b.free()
     ctx.close()
 
 
@@ -267,7 +297,7 @@ def test_eight_byte_messages_for_the_128_byte_families(oracle, algo):
             got, _ = H.run_allreduce(ctx, algo, ins, transport=WIRE, inplace=inplace)
             H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
     with pytest.raises(vr.VRError):
-        ctx.set_tuning(wire_fenced=3)
+        ctx.set_tuning(wire_fenced=5)
     ctx.close()
 
 
