@@ -101,6 +101,8 @@ def lib():
         "vr_ctx_get_tuning": (i, [vp, C.c_char_p, C.POINTER(i)]),
         "vr_time_allreduce": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_allgather": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
+        "vr_time_allreduce_kernel": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
+        "vr_time_allgather_kernel": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
         "vr_time_copy": (i, [vp, vp, vp, vp, sz, i, C.POINTER(C.c_float)]),
         "vr_stream_probe": (i, [vp, vp, i, vp, vp, sz]),
         "vr_stream_probe_multi": (i, [vp, vp, vpp, vpp, sz]),
@@ -386,6 +388,23 @@ class VirtualRanks:
         self._reserve_for(algo, transport)
         _check(lib().vr_time_allreduce(self._h, stream, algo_id(algo), transport, _table(bufs),
                                        _table(outs) if outs is not None else None, nelems, iters, ms))
+        return np.frombuffer(ms, np.float32).copy()
+
+    def time_allreduce_kernel(self, algo, bufs, nelems, iters, outs=None, transport=TRANSPORT_DEFAULT,
+                              stream=None):
+        """Kernel execution time of each launch (ms), from events attached to the dispatches."""
+        ms = (C.c_float * iters)()
+        self._reserve_for(algo, transport)
+        _check(lib().vr_time_allreduce_kernel(self._h, stream, algo_id(algo), transport, _table(bufs),
+                                              _table(outs) if outs is not None else None, nelems, iters, ms))
+        return np.frombuffer(ms, np.float32).copy()
+
+    def time_allgather_kernel(self, algo, inputs, outputs, nelems, iters, transport=TRANSPORT_DEFAULT,
+                              stream=None):
+        ms = (C.c_float * iters)()
+        self._reserve_for(algo, transport)
+        _check(lib().vr_time_allgather_kernel(self._h, stream, algo_id(algo), transport, _table(inputs),
+                                              _table(outputs), nelems, iters, ms))
         return np.frombuffer(ms, np.float32).copy()
 
     def time_allreduce_grouped(self, algo, bufs, nelems, groups, per_group, outs=None,

@@ -8,6 +8,7 @@
 #include <time.h>
 
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "vr_host.h"
@@ -686,6 +687,73 @@ extern "C" int vr_time_allgather(vr_ctx *ctx, void *stream, int algo, int transp
   });
 }
 
+// Per-launch kernel execution times from events attached to the dispatches
+// themselves: what a kernel trace shows, measured in the running program.
+template <typename F>
+static int time_kernels_attached(hipStream_t s, int iters, float *ms_out, F &&launch) {
+  if (iters <= 0 || !ms_out) return fail(VR_ERR_INVALID, "iters <= 0 or null ms_out");
+  const int kBatch = 128;
+  std::vector<hipEvent_t> ev(2 * (size_t)kBatch, nullptr);
+  int rc = VR_OK;
+  for (auto &e : ev)
+    if (hipError_t err = hipEventCreate(&e); err != hipSuccess) { rc = fail_hip(err, "hipEventCreate"); break; }
+  for (int done = 0; done < iters && rc == VR_OK; done += kBatch) {
+    const int n = (iters - done < kBatch) ? iters - done : kBatch;
+    for (int i = 0; i < n && rc == VR_OK; ++i) {
+      tl_kernel_events.start = ev[2 * i];
+      tl_kernel_events.stop = ev[2 * i + 1];
+      rc = launch();
+      tl_kernel_events = KernelEvents();
+    }
+    if (rc != VR_OK) break;
+    if (hipError_t e = hipStreamSynchronize(s); e != hipSuccess) { rc = fail_hip(e, "hipStreamSynchronize"); break; }
+    for (int i = 0; i < n; ++i) {
+      float ms = 0.f;
+      if (hipError_t e = hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]); e != hipSuccess) {
+        rc = fail_hip(e, "hipEventElapsedTime (kernel-attached events)");
+        break;
+      }
+      ms_out[done + i] = ms;
+    }
+  }
+  tl_kernel_events = KernelEvents();
+  for (auto &e : ev)
+    if (e) (void)hipEventDestroy(e);
+  return rc;
+}
+
+extern "C" int vr_time_allreduce_kernel(vr_ctx *ctx, void *stream, int algo, int transport,
+                                        void *const bufs[], void *const outs[], size_t nelems,
+                                        int iters, float *ms_out) {
+  Prepared p;
+  if (int rc = prepare_allreduce(ctx, algo, bufs, outs, nelems, &p)) return rc;
+  int tr;
+  if (int rc = resolve_transport(p.a, transport, &tr)) return rc;
+  const Tuning t = tuning_for(ctx, p.a, p.bytes_all_ranks, p.bytes_all_ranks, p.in_place);
+  hipStream_t s = (hipStream_t)stream;
+  return time_kernels_attached(s, iters, ms_out, [&]() -> int {
+    uint32_t next = ctx->seq_no;
+    int rc = run_allreduce(ctx, s, p, tr, t, ctx->seq_no, 0, &next);
+    ctx->seq_no = next;
+    return rc;
+  });
+}
+
+extern "C" int vr_time_allgather_kernel(vr_ctx *ctx, void *stream, int algo, int transport,
+                                        const void *const inputs[], void *const outputs[],
+                                        size_t nelems, int iters, float *ms_out) {
+  PreparedGather p;
+  if (int rc = prepare_allgather(ctx, algo, inputs, outputs, nelems, &p)) return rc;
+  const Tuning t = allgather_tuning(ctx, p.a, nelems);
+  hipStream_t s = (hipStream_t)stream;
+  return time_kernels_attached(s, iters, ms_out, [&]() -> int {
+    uint32_t next = ctx->seq_no;
+    int rc = run_allgather(ctx, s, p, transport, t, nelems, ctx->seq_no, 0, &next);
+    ctx->seq_no = next;
+    return rc;
+  });
+}
+
 // `groups` event pairs, each around `per_group` back-to-back vr_allreduce calls made
 // exactly as a caller makes them (validation, launch heuristics and launch in every
 // call).  ms_out[g] = device time of group g divided by per_group; *host_call_us
@@ -876,9 +944,9 @@ extern "C" void vr_generate(uint16_t *host_buf, size_t n, uint64_t seed, int dis
   vr_generate_dt(VR_DTYPE_F16, host_buf, n, seed, dist, p0, p1);
 }
 
-extern "C" void vr_generate_dt(int dtype, uint16_t *host_buf, size_t n, uint64_t seed, int dist,
-                               double p0, double p1) {
-  for (size_t i = 0; i < n; ++i) {
+static void generate_range(int dtype, uint16_t *host_buf, size_t begin, size_t end, uint64_t seed, int dist,
+                           double p0, double p1) {
+  for (size_t i = begin; i < end; ++i) {
     const uint64_t z0 = splitmix64_at(seed, 2 * (uint64_t)i);
     const uint64_t z1 = splitmix64_at(seed, 2 * (uint64_t)i + 1);
     double x;
@@ -891,6 +959,28 @@ extern "C" void vr_generate_dt(int dtype, uint16_t *host_buf, size_t n, uint64_t
     }
     host_buf[i] = f64_to_elem(dtype, x);
   }
+}
+
+// Element i depends on (seed, i) only, so large buffers are filled by several
+// host threads, each on a contiguous range; the result does not depend on how
+// many there are.
+extern "C" void vr_generate_dt(int dtype, uint16_t *host_buf, size_t n, uint64_t seed, int dist,
+                               double p0, double p1) {
+  size_t threads = n >> 20;                           // at least 1 Mi elements per thread
+  const size_t hw = std::thread::hardware_concurrency();
+  if (threads > hw) threads = hw;
+  if (threads > 16) threads = 16;
+  if (threads <= 1) {
+    generate_range(dtype, host_buf, 0, n, seed, dist, p0, p1);
+    return;
+  }
+  std::vector<std::thread> pool;
+  const size_t per = (n + threads - 1) / threads;
+  for (size_t t = 0; t < threads; ++t) {
+    const size_t b = t * per, e = b + per < n ? b + per : n;
+    if (b < e) pool.emplace_back(generate_range, dtype, host_buf, b, e, seed, dist, p0, p1);
+  }
+  for (auto &th : pool) th.join();
 }
 
 extern "C" int vr_parse_nelems(const char *text, size_t *out) {

@@ -21,9 +21,13 @@
 // reference predicates its tail wire per lane, rt64_128.hpp:570-582), and the
 // cache-policy bits of each access are chosen per launch.
 
+#include <hip/hip_ext.h>
+
 #include "vr_internal.h"
 
 namespace vr {
+
+thread_local KernelEvents tl_kernel_events;
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
@@ -295,10 +299,15 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
     const size_t seg = chunk_bytes - off < seg_max ? chunk_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
     const dim3 grid(bpr * N), block(t.block);
+    // kernel-attached profiling events: start on the first segment, stop on the last
+    hipEvent_t ev0 = off == 0 ? tl_kernel_events.start : nullptr;
+    hipEvent_t ev1 = off + seg >= chunk_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
-      hipLaunchKernelGGL((k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value,
-                                             decltype(st_aux)::value>),
-                         grid, block, 0, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+      auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
+      if (ev0 || ev1)
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+      else
+        hipLaunchKernelGGL(kernel, grid, block, 0, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
@@ -372,9 +381,14 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
     const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
     const dim3 grid(bpr * N), block(t.block);
+    hipEvent_t ev0 = off == 0 ? tl_kernel_events.start : nullptr;
+    hipEvent_t ev1 = off + seg >= slice_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
-      hipLaunchKernelGGL((k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>),
-                         grid, block, 0, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+      auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
+      if (ev0 || ev1)
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+      else
+        hipLaunchKernelGGL(kernel, grid, block, 0, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;

@@ -50,6 +50,16 @@ struct DeviceInfo {
   char arch[64] = {0};
 };
 
+// Events to attach to the next collective's kernel dispatches on this host thread
+// (hipExtLaunchKernel): `start` is stamped when the first kernel of the collective
+// begins to execute, `stop` when its last kernel ends, from the dispatches' own
+// timestamps, the counterpart of the reference's SYCL event profiling
+// (main.cpp:36-43).  Both null (the default): plain launches.
+struct KernelEvents {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local KernelEvents tl_kernel_events;
+
 // Direct transport -----------------------------------------------------------
 // in/out hold nranks pointers; chunk_elems = nelems / nranks; vec_halves is 8
 // (16-byte accesses) or 4 (8-byte accesses, for chunks or pointers that are only

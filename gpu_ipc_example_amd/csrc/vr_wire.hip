@@ -31,6 +31,8 @@
 // another wave has given up) a wave records a time-out in the status word and
 // runs to completion without waiting again, so the grid always drains.
 
+#include <hip/hip_ext.h>
+
 #include <mutex>
 #include <unordered_map>
 
@@ -1453,6 +1455,8 @@ hipError_t launch_wire(hipStream_t s, WireFlow flow, WireFormat fmt, int vec_hal
   void *kargs[] = {&args};
   const dim3 grid(blocks), block(block_threads);
   if (cooperative) return hipLaunchCooperativeKernel(fn, grid, block, kargs, 0, s);
+  if (tl_kernel_events.start || tl_kernel_events.stop)
+    return hipExtLaunchKernel(fn, grid, block, kargs, 0, s, tl_kernel_events.start, tl_kernel_events.stop, 0);
   return hipLaunchKernel(fn, grid, block, kargs, 0, s);
 }
 

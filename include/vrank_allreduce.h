@@ -343,6 +343,17 @@ int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);
  * times in milliseconds (ms_out[iters]).  Out-of-place when outs != NULL. */
 int vr_time_allreduce(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
                       void *const outs[], size_t nelems, int iters, float *ms_out);
+/* Per-launch kernel EXECUTION times in milliseconds, from events attached to the
+ * kernel dispatches themselves (their own begin / end timestamps, what a kernel
+ * trace shows and what the reference prints from its SYCL event, main.cpp:36-43);
+ * no host or event-command overhead is included.  A collective that takes several
+ * kernels (chunks above 1 GiB) is timed from the first one's begin to the last
+ * one's end. */
+int vr_time_allreduce_kernel(vr_ctx *ctx, void *stream, int algo, int transport, void *const bufs[],
+                             void *const outs[], size_t nelems, int iters, float *ms_out);
+int vr_time_allgather_kernel(vr_ctx *ctx, void *stream, int algo, int transport,
+                             const void *const inputs[], void *const outputs[], size_t nelems,
+                             int iters, float *ms_out);
 /* `groups` event pairs, each around `per_group` back-to-back vr_allreduce calls made
  * exactly as a caller makes them.  ms_out[g] = device time of group g / per_group;
  * *host_call_us (optional) = host wall time one vr_allreduce call takes to return

@@ -36,3 +36,31 @@ def test_measured_traffic_constants_are_the_numbers_in_the_profiles():
         assert "{:,} B".format(nbytes) in text, (workload, transport, nbytes, fname)
     assert bench.measured_traffic("cfg3", "default") == bench.MEASURED_TRAFFIC_BYTES[("cfg3", "direct")][0]
     assert bench.measured_traffic("cfg3", "wire") == bench.MEASURED_TRAFFIC_BYTES.get(("cfg3", "wire"), (None,))[0]
+
+
+def test_default_line_carries_the_fixed_sample_and_the_other_configurations():
+    """The driver's one line must hold: a kernel-time sample whose size does not depend
+    on --steps, the in-place figure on cold sets, config 4, config 5 at three sizes
+    and the latency figures measured on the C side.  Checked on the source, so that
+    no GPU is needed: every key is one the default path writes."""
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.KERNEL_SAMPLE_LAUNCHES >= 200 and bench.KERNEL_SAMPLE_MIN_PAIRS >= 20
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    for key in ("kernel_us_min", "kernel_us_p50", "kernel_us_p99", "n_pairs", "in_place_cold",
+                "cfg4_allgather", "cfg5_sweep_points", "latency_1MiB_per_rank", "host_call_us",
+                "back_to_back_us_per_launch", "kernel_trace_p50_us", "same_buffers_cache_warm",
+                "hbm_ceilings", "cpu_baseline", "roofline"):
+        assert '"%s"' % key in src, key
+    us, fname = bench.CFG2_KERNEL_TRACE
+    text = open(os.path.join(ROOT, "profiles", fname)).read()
+    assert ("%.2f" % us) in text, (us, fname)
+
+
+def test_tiled_inputs_are_the_same_on_both_sides():
+    """Workloads above 16 Mi elements per rank repeat a 16 Mi-element draw; the GPU side
+    (setup) and the CPU side (cpu_leg) must build the same arrays."""
+    sys.path.insert(0, ROOT)
+    import bench
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    assert src.count("min(ne, 1 << 24)") == 2
