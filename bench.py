@@ -652,10 +652,11 @@ def main():
             "note": "one buffer set, cached loads: inputs served by the Infinity Cache; "
                     "not an HBM figure"}
 
-    if name == "cfg3" and not args.only_headline:
-        result["latency_1MiB_per_rank"] = latency_block(vr, binding, want_check, gpu_results, args.latency_iters)
+    if not args.only_headline and (name == "cfg3" or reduces):
+        if name == "cfg3":
+            result["latency_1MiB_per_rank"] = latency_block(vr, binding, want_check, gpu_results, args.latency_iters)
         result["hbm_ceilings"] = hbm_ceilings(binding, ctx)
-        if sets[0][1] is not None and reduces:
+        if sets[0][1] is not None and reduces and TRANSPORT != vr.TRANSPORT_WIRE and algo != "parallel":
             # the same kernel, grid and policies without the adds, on the same buffer sets
             time_kernels(binding, ctx, name, sets, 8)                      # back to steady state
             c_ms = multi_stream_copy(binding, ctx, name, sets, 100, 10)
@@ -665,12 +666,13 @@ def main():
                 "allreduce_us_avg_same_run": round(a_ms * 1e3, 3),
                 "note": "k_direct_allreduce with the adds removed: %d read + %d write streams, same "
                         "grid, buffer addressing and nt / nt sc1 policies, same rotating buffer sets" % (n, n)}
-        # free the headline's 2 GiB before the other configurations allocate theirs
-        for ins, outs in sets:
-            for b in ins + (outs or []):
-                b.free()
-        result["cfg4_allgather"] = allgather_block(vr, binding, want_check, gpu_results)
-        result["cfg5_sweep_points"] = cfg5_block(vr, binding)
+        if name == "cfg3":
+            # free the headline's 2 GiB before the other configurations allocate theirs
+            for ins, outs in sets:
+                for b in ins + (outs or []):
+                    b.free()
+            result["cfg4_allgather"] = allgather_block(vr, binding, want_check, gpu_results)
+            result["cfg5_sweep_points"] = cfg5_block(vr, binding)
 
     if want_check:
         result["cpu_baseline"], bad = cpu_leg(name, gpu_results, args.cpu_seconds)

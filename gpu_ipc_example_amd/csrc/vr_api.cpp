@@ -378,6 +378,11 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // trip's loads and its stores shortens the launch by 2.5 % at 8 ranks (0.5 %
       // at 4; it costs 1-2 % at 2 and 16 ranks and 8 % when the data is cache-resident).
       t.f16_wide = ctx->nranks == 4 || ctx->nranks == 8;
+      // Eight ranks with chunks of 16 MiB and more (128 MiB per rank and up): one
+      // launch per 4 MiB of every chunk, the shape of the 32 MiB-per-rank launch,
+      // measured 5 % (128 MiB per rank) to 9 % (256 MiB) faster than one long
+      // launch; no gain at 4 or 16 ranks, a loss at 2.
+      if (ctx->nranks == 8 && read_bytes / 64 >= ((size_t)16 << 20)) t.segment_bytes = (size_t)4 << 20;
     }
   }
   const TuningOverrides &o = ctx->tune;

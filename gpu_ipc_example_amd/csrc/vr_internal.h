@@ -105,6 +105,8 @@ struct WireArgs {
   int rank_first, rank_count; // the grid holds the wires of ranks [rank_first, rank_first + rank_count):
                              // block b is rank rank_first + b % rank_count (all ranks: 0, N)
   uint32_t stream_io;        // 1: inputs are loaded and outputs stored with streaming cache policies
+  uint32_t io_narrow;        // 1: this launch's inputs / outputs are only 8-byte aligned: a lane's 16 bytes
+                             //    travel as two 8-byte accesses (the messages are the same)
   uint32_t *status;          // non-zero once any poll gave up
 };
 

@@ -70,28 +70,42 @@ static __device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_rsrc(const void *p
 typedef unsigned int io_u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int io_u32x4 __attribute__((ext_vector_type(4)));
 
-static __device__ __forceinline__ uint32_t io_ld32(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
-  return nt ? __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoStreamLoad)
-            : __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoCached);
+// `io`: bit 0 = streaming cache policy (nt loads, nt sc1 stores) instead of cached
+// accesses; bit 1 = the launch's inputs / outputs are only 8-byte aligned, so a
+// lane's 16 bytes travel as two 8-byte accesses (same registers, same messages).
+constexpr uint32_t kIoStream = 1u, kIoNarrow = 2u;
+
+static __device__ __forceinline__ uint32_t io_ld32(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t io) {
+  return (io & kIoStream) ? __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoStreamLoad)
+                          : __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, kIoCached);
 }
-static __device__ __forceinline__ io_u32x2 io_ld64(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
-  return nt ? __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoStreamLoad)
-            : __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoCached);
+static __device__ __forceinline__ io_u32x2 io_ld64(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t io) {
+  return (io & kIoStream) ? __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoStreamLoad)
+                          : __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, kIoCached);
 }
-static __device__ __forceinline__ io_u32x4 io_ld128(__amdgpu_buffer_rsrc_t rs, uint32_t off, bool nt) {
-  return nt ? __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoStreamLoad)
-            : __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoCached);
+static __device__ __forceinline__ io_u32x4 io_ld128(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t io) {
+  if (io & kIoNarrow) {
+    const io_u32x2 lo = io_ld64(rs, off, io), hi = io_ld64(rs, off + 8u, io);
+    return io_u32x4{lo.x, lo.y, hi.x, hi.y};
+  }
+  return (io & kIoStream) ? __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoStreamLoad)
+                          : __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, kIoCached);
 }
-static __device__ __forceinline__ void io_st32(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t v, bool nt) {
-  if (nt) __builtin_amdgcn_raw_buffer_store_b32(v, rs, off, 0, kIoStreamStore);
+static __device__ __forceinline__ void io_st32(__amdgpu_buffer_rsrc_t rs, uint32_t off, uint32_t v, uint32_t io) {
+  if (io & kIoStream) __builtin_amdgcn_raw_buffer_store_b32(v, rs, off, 0, kIoStreamStore);
   else __builtin_amdgcn_raw_buffer_store_b32(v, rs, off, 0, kIoCached);
 }
-static __device__ __forceinline__ void io_st64(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x2 v, bool nt) {
-  if (nt) __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kIoStreamStore);
+static __device__ __forceinline__ void io_st64(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x2 v, uint32_t io) {
+  if (io & kIoStream) __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kIoStreamStore);
   else __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kIoCached);
 }
-static __device__ __forceinline__ void io_st128(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x4 v, bool nt) {
-  if (nt) __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kIoStreamStore);
+static __device__ __forceinline__ void io_st128(__amdgpu_buffer_rsrc_t rs, uint32_t off, io_u32x4 v, uint32_t io) {
+  if (io & kIoNarrow) {
+    io_st64(rs, off, io_u32x2{v.x, v.y}, io);
+    io_st64(rs, off + 8u, io_u32x2{v.z, v.w}, io);
+    return;
+  }
+  if (io & kIoStream) __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kIoStreamStore);
   else __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kIoCached);
 }
 
@@ -163,7 +177,7 @@ struct WireLL {
     uint32_t d[U];
   };
 
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, uint32_t nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
@@ -171,7 +185,7 @@ struct WireLL {
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
-                                               bool nt) {
+                                               uint32_t nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) io_st32(rs, (u * 64u + lane) * 4u, r.d[u], nt);
@@ -277,7 +291,7 @@ struct WireLL16 {
   static __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const char *slot) {
     return wave_rsrc(slot, kSlotBytes);
   }
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, uint32_t nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
@@ -289,7 +303,7 @@ struct WireLL16 {
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
-                                               bool nt) {
+                                               uint32_t nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -400,7 +414,7 @@ struct WireRt128 {
   static __device__ __forceinline__ uint32_t io_off(int u, uint32_t lane) {
     return (lane & 15u) == 15u ? kOffNowhere : (uint32_t)u * 480u + (lane >> 4) * 120u + (lane & 15u) * 8u;
   }
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, uint32_t nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
@@ -412,7 +426,7 @@ struct WireRt128 {
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
-                                               bool nt) {
+                                               uint32_t nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -533,7 +547,7 @@ struct WireRt256 {
   static __device__ __forceinline__ uint32_t io_off(int u, uint32_t lane) {
     return (lane & 15u) == 15u ? kOffNowhere : (uint32_t)u * 960u + (lane >> 4) * 240u + (lane & 15u) * 16u;
   }
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, uint32_t nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
@@ -547,7 +561,7 @@ struct WireRt256 {
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
-                                               bool nt) {
+                                               uint32_t nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -683,7 +697,7 @@ struct WireFlag {
     V d[U];
   };
 
-  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, bool nt) {
+  static __device__ __forceinline__ Reg load(const char *p, uint32_t left, uint32_t lane, uint32_t nt) {
     Reg r;
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
@@ -695,7 +709,7 @@ struct WireFlag {
     return r;
   }
   static __device__ __forceinline__ void store(char *p, uint32_t left, uint32_t lane, const Reg &r,
-                                               bool nt) {
+                                               uint32_t nt) {
     const __amdgpu_buffer_rsrc_t rs = wave_rsrc(p, left);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -850,7 +864,7 @@ struct Sinks {
   const uint32_t wid = (blockIdx.x / held) * (blockDim.x >> 6) + (threadIdx.x >> 6); \
   if (wid >= a.waves_per_rank) return;                                               \
   Spin spin{a.spin_limit, a.status, lane, false};                                    \
-  const bool nt = a.stream_io != 0;                                                  \
+  const uint32_t nt = (a.stream_io ? kIoStream : 0u) | (a.io_narrow ? kIoNarrow : 0u);  \
   const size_t chunk = a.chunk_bytes
 
 static __device__ __forceinline__ uint32_t bytes_left(size_t chunk, size_t off, uint32_t wire) {

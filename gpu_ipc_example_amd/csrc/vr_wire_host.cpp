@@ -95,19 +95,33 @@ struct WireLaunch {
   uint32_t *status;
   int first, count;       // the launch holds the wires of ranks [first, first + count)
   bool always_clear;      // clear the sinks before every launch (fixed scratch shared by contexts)
+  bool io_narrow = false; // inputs / outputs of this launch are only 8-byte aligned
 };
+
+// How the Rt64_128 families synchronise (the "wire_fenced" setting).  Left to the
+// library, the all-to-all flows (ParallelTransmit, BisectPTransmit, SimpleTransmit)
+// take flag words with agent-scope accesses ordered by store completion: as fast as
+// or faster than the reference's embedded-flag messages at every size measured, and
+// resting on nothing but the scope semantics of the accesses.  The neighbour-ring and
+// sequential flows keep the reference's messages, which are up to 15 % faster there.
+static int flag_word_mode(const vr_ctx *c, const AlgoInfo *a) {
+  if (c->tune.wire_fenced >= 0) return c->tune.wire_fenced;
+  if (a->allgather) return 0;
+  return (a->transmit == T_PARALLEL || a->transmit == T_BISECT || a->transmit == T_SIMPLE) ? 4 : 0;
+}
 
 // Wire format of an algo under the context's settings.  `vec_halves` = 8 says that
 // every pointer and the chunk allow 16-byte accesses.
 static WireFormat format_for(const vr_ctx *c, const AlgoInfo *a, size_t chunk_bytes, int vec_halves) {
   WireFormat fmt = a->wire_format();
   const bool big = fmt == WIRE_FMT_RT128 || fmt == WIRE_FMT_RT256;
-  if (big && c->tune.wire_fenced == 1) fmt = WIRE_FMT_FLAG;
+  const int fenced = flag_word_mode(c, a);
+  if (big && fenced == 1) fmt = WIRE_FMT_FLAG;
   // Self-validating 8-byte messages for the Rt64_128 families too: nothing beyond
   // 8-byte store atomicity is assumed, at half the payload per message.
-  if (big && c->tune.wire_fenced == 2) fmt = WIRE_FMT_LL;
-  if (big && c->tune.wire_fenced == 3) fmt = WIRE_FMT_FLAG_WT;
-  if (big && c->tune.wire_fenced == 4) fmt = WIRE_FMT_FLAG_SCOPED;
+  if (big && fenced == 2) fmt = WIRE_FMT_LL;
+  if (big && fenced == 3) fmt = WIRE_FMT_FLAG_WT;
+  if (big && fenced == 4) fmt = WIRE_FMT_FLAG_SCOPED;
   if (fmt == WIRE_FMT_LL16 && c->tune.wire_msg16 == 0) fmt = WIRE_FMT_LL;
   // `parallel` names the transmit, not a wire format: it takes the reference's
   // 256-byte messages (16 bytes per lane) when every pointer and the chunk allow
@@ -117,15 +131,18 @@ static WireFormat format_for(const vr_ctx *c, const AlgoInfo *a, size_t chunk_by
   return fmt;
 }
 
-// Does the algo's wire format, as the context is set, move 16 bytes per lane when
-// the chunk allows it (and therefore need 16-byte aligned buffers then)?  The
-// 8-byte-message formats (Rt64, Rt64_128) and the 16-byte-message formats (whose
-// calcWorkSize already demands 16-byte alignment) do not depend on it.
+// Does the algo's wire format, as the context is set, carry 16 bytes per lane when
+// the chunk is a multiple of 16 bytes?  (Then every rank must decide so from the
+// element count alone; a rank whose buffers are only 8-byte aligned moves each
+// lane's 16 bytes as two 8-byte accesses.)  The 8-byte-message formats (Rt64,
+// Rt64_128) and the 16-byte-message formats (whose calcWorkSize already demands
+// 16-byte alignment) do not depend on it.
 static bool format_widens_with_alignment(const vr_ctx *c, const AlgoInfo *a) {
   if (a == &kAlgos[VR_ALGO_PARALLEL]) return true;
   const WireFormat fmt = a->wire_format();
   const bool big = fmt == WIRE_FMT_RT128 || fmt == WIRE_FMT_RT256;
-  return big && (c->tune.wire_fenced == 1 || c->tune.wire_fenced == 3 || c->tune.wire_fenced == 4);
+  const int fenced = flag_word_mode(c, a);
+  return big && (fenced == 1 || fenced == 3 || fenced == 4);
 }
 
 // Shape of one wire-transport launch: which kernel, how many wires per rank, how
@@ -267,6 +284,7 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
   args.spin_limit = limit > 0xffffffffull ? 0xffffffffu : (uint32_t)limit;
   args.status = wlch.status;
   args.ahead = c->tune.wire_ahead > 0 ? (uint32_t)c->tune.wire_ahead : kWireAhead;
+  args.io_narrow = wlch.io_narrow ? 1u : 0u;
   args.rank_first = wlch.first;
   args.rank_count = wlch.count;
   // Inputs and outputs that cannot stay in the 256 MiB memory-side cache anyway are
@@ -463,6 +481,7 @@ static int allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first, int c
   memset(&out, 0, sizeof out);
   size_t work = 0;
   int vec_halves = a->msg_bytes == 16 ? 8 : 4;
+  bool narrow = false;
   for (int i = 0; i < count; ++i) {
     void *input = inputs[i], *output = outputs && outputs[i] ? outputs[i] : inputs[i];
     // calcWorkSize sees one rank's pointers at a time
@@ -473,12 +492,8 @@ static int allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first, int c
     if (int rc = vr_check_allreduce(algo, N, table, nelems, &work)) return rc;
     if (ranges_partially_overlap(output, input, nelems * 2))
       return fail(VR_ERR_OVERLAP, "output partially overlaps input");
-    if (widens && (work / 2) % 8 == 0) {
-      vec_halves = 8;
-      if ((uintptr_t)input % 16 || (uintptr_t)output % 16)
-        return fail(VR_ERR_UNALIGNED, std::string(a->name) + " moves a chunk that is a multiple of 16 bytes with "
-                                          "16-byte accesses on every rank: input and output must be 16-byte aligned");
-    }
+    if (widens && (work / 2) % 8 == 0) vec_halves = 8;
+    if ((uintptr_t)input % 16 || (uintptr_t)output % 16) narrow = true;
     in.p[first + i] = input;
     out.p[first + i] = output;
   }
@@ -487,7 +502,7 @@ static int allreduce_ranks(vr_ctx *ctx, void *stream, int algo, int first, int c
   vr_geometry geom;
   if (int rc = vr_launch_geometry(algo, N, nelems, &geom)) return rc;
   if (int rc = admit_group_launch(ctx, k.scatter[0], stream, first, count, *seq_no)) return rc;
-  const WireLaunch wlch = {&k, nullptr, ctx->status, first, count, false};
+  const WireLaunch wlch = {&k, nullptr, ctx->status, first, count, false, narrow};
   uint32_t seq = *seq_no, used = 0;
   if (int rc = wire_launch(ctx, (hipStream_t)stream, a, in, out, work, vec_halves, &seq, user_wires, &used,
                            wlch))

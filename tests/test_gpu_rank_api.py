@@ -162,6 +162,8 @@ def test_sink_bytes_are_the_reference_messages(ranks, oracle, algo):
     assert cap * 4 * msgs == wire_bytes and size * 4 * msgs == 2048
     R = ranks[2]
     R.zero()
+    for c in R.ctx:
+        c.set_tuning(wire_fenced=0)        # the reference's messages (left alone, ParallelTransmit takes flag words)
     wires = 5                                          # wires per chunk, the last one ragged
     chunk_bytes = wire_bytes * (wires - 1) + 16 * 7
     n = 2 * chunk_bytes // 2
@@ -190,6 +192,8 @@ def test_sink_bytes_are_the_reference_messages(ranks, oracle, algo):
         slot = (x_id + 1) * 8 + 0                      # owner rank 1 gathers into rank 0
         got_slot = gath0[slot * 512:(slot + 1) * 512]
         assert np.array_equal(got_slot, expect_slot(want[half:], w)), (algo, "gather", w)
+    for c in R.ctx:
+        c.set_tuning(wire_fenced=-1)
 
 
 def test_rank_call_validates_like_the_constructor(ranks):
@@ -213,38 +217,48 @@ def test_rank_call_validates_like_the_constructor(ranks):
     with pytest.raises(vr.VRError) as e:
         c.allreduce_rank("simple", 0, buf.ptr, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 0)
     assert e.value.code == "INVALID"
-    # `parallel` (256-byte messages) moves a chunk of 16-byte multiples with 16-byte
-    # accesses on every rank; the 8-byte-message protocols accept what calcWorkSize
-    # accepts (allreduce.hpp:110: alignment to message_t), see the next test
+    # the 16-byte-message protocols demand 16-byte alignment (rt64.hpp:3-20 message_t)
     with pytest.raises(vr.VRError) as e:
-        c.allreduce_rank("parallel", 0, buf.ptr + 8, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 1)
-    assert e.value.code == "UNALIGNED" and "16-byte" in e.value.detail
+        c.allreduce_rank("simple_ring", 0, buf.ptr + 8, s0[0], s1[0], s0, s1, R.sink_bytes, 64, 1)
+    assert e.value.code == "UNALIGNED"
     buf.free()
 
 
-@pytest.mark.parametrize("algo", ["simple", "bisect", "small", "simple_transmit"])
-def test_eight_byte_aligned_buffers_with_sixteen_byte_chunks(ranks, oracle, algo):
+@pytest.mark.parametrize("fenced", [-1, 0])
+@pytest.mark.parametrize("algo", ["simple", "bisect", "small", "simple_transmit", "parallel"])
+def test_eight_byte_aligned_buffers_with_sixteen_byte_chunks(ranks, oracle, algo, fenced):
     """message_t of small / simple / bisect is 8 bytes (rt64.hpp:335, rt64_128.hpp:539):
     an 8-byte-aligned buffer is accepted whatever the chunk length, as by the
-    reference's per-rank calcWorkSize."""
+    reference's per-rank calcWorkSize, with the reference's messages (fenced 0) and
+    with flag words (the library's choice), also when only some ranks' buffers are
+    off a 16-byte boundary."""
     R = ranks[4]
     R.zero()
+    for c in R.ctx:
+        c.set_tuning(wire_fenced=fenced)
     seq = 1
-    for n in (4 * 64, 4 * 8 * 1001):                     # chunks of 16-byte multiples
+    for n, odd_ranks in ((4 * 64, (0, 1, 2, 3)), (4 * 8 * 1001, (0, 1, 2, 3)), (4 * 8 * 333, (1, 2))):
         ins = H.make_inputs(oracle, 4, n, 8700 + n)
-        src = H.RankBuffers(4, n, 8)                     # every buffer 8 bytes off a 16-byte boundary
-        src.upload(ins)
+        off = [8 if r in odd_ranks else 16 for r in range(4)]     # 8 bytes off a 16-byte boundary, or on one
+        bufs = [DeviceBuffer(n * 2 + 64) for _ in range(4)]
+        for r in range(4):
+            bufs[r].upload(ins[r], off[r])
+        ptrs = [bufs[r].ptr + off[r] for r in range(4)]
         s0 = [b.ptr for b in R.scatter]
         s1 = [b.ptr for b in R.gather]
         nxt = seq
         for r in range(4):
-            nxt = R.ctx[r].allreduce_rank(algo, r, src.ptrs[r], s0[r], s1[r], s0, s1, R.sink_bytes, n, seq,
+            nxt = R.ctx[r].allreduce_rank(algo, r, ptrs[r], s0[r], s1[r], s0, s1, R.sink_bytes, n, seq,
                                           stream=R.handle(r))
         for r in range(4):
             R.ctx[r].check(R.handle(r))
         seq = nxt
-        H.assert_all_ranks_equal(oracle, src.download(), H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
-        src.free()
+        got = [bufs[r].download(np.uint16, n, off[r]) for r in range(4)]
+        H.assert_all_ranks_equal(oracle, got, H.expected(oracle, algo, ins), "%s n=%d" % (algo, n))
+        for b in bufs:
+            b.free()
+    for c in R.ctx:
+        c.set_tuning(wire_fenced=-1)
 
 
 class Groups:

@@ -174,9 +174,16 @@ def test_poll_timeout_is_reported_and_recoverable(ctxs, oracle):
     ctx.close()
 
 
-def test_config3_bisect_32mib_wire(ctxs, oracle):
+@pytest.mark.parametrize("fenced", [-1, 0])
+def test_config3_bisect_32mib_wire(ctxs, oracle, fenced):
+    """The headline shape through scratch: flag words (the library's choice) and the
+    reference's 128-byte messages."""
     ins = H.make_inputs(oracle, 8, 16777216, 3000, DIST_NORMAL, 0.0, 0.02)
-    got, _ = H.run_allreduce(ctxs[8], "bisect", ins, transport=WIRE)
+    ctxs[8].set_tuning(wire_fenced=fenced)
+    try:
+        got, _ = H.run_allreduce(ctxs[8], "bisect", ins, transport=WIRE)
+    finally:
+        ctxs[8].set_tuning(wire_fenced=-1)
     H.assert_all_ranks_equal(oracle, got, oracle.bisect(ins))
 
 
@@ -188,15 +195,20 @@ def test_parallel_defaults_to_wire_and_sweep_sizes(ctxs, oracle):
         H.assert_all_ranks_equal(oracle, got, oracle.rotated(ins), "n=%d" % n)
 
 
-@pytest.mark.parametrize("log2_elems", [24, 25, 26, 27])
-def test_config5_parallel_large_sizes(ctxs, oracle, log2_elems):
+@pytest.mark.parametrize("log2_elems,fenced", [(24, -1), (25, -1), (26, -1), (27, -1), (24, 0), (27, 0)])
+def test_config5_parallel_large_sizes(ctxs, oracle, log2_elems, fenced):
     """The sweep's named protocol on its default (wire) transport at 32, 64, 128 and
     256 MiB per rank: N(0,1) inputs, rank 0 compared in full with the rotated-order
-    oracle, the other ranks by equality with rank 0."""
+    oracle, the other ranks by equality with rank 0.  With the library's own choice of
+    format (flag words) and with the reference's 256-byte messages (fenced 0)."""
     n = 1 << log2_elems
     ins = H.make_inputs(oracle, 8, n, 5000 + log2_elems)
     want = oracle.rotated(ins)
-    got, _ = H.run_allreduce(ctxs[8], "parallel", ins)          # default transport = wire
+    ctxs[8].set_tuning(wire_fenced=fenced)
+    try:
+        got, _ = H.run_allreduce(ctxs[8], "parallel", ins)          # default transport = wire
+    finally:
+        ctxs[8].set_tuning(wire_fenced=-1)
     assert oracle.count_mismatch(got[0], want) == 0, n
     for r in range(1, 8):
         assert oracle.count_mismatch(got[r], got[0]) == 0, (n, r)
@@ -239,14 +251,15 @@ def test_allgather_wire(ctxs, oracle, nranks, algo):
                 assert (got[r] == want).all(), (n, r, alias)
 
 
-@pytest.mark.parametrize("fenced", [1, 3, 4])
+@pytest.mark.parametrize("fenced", [0, 1, 3, 4])
 @pytest.mark.parametrize("algo", ["simple", "parallel", "bisect", "simple_ring", "simple_pcie",
                                   "simple_pcie_p", "simple_transmit"])
 def test_fenced_flag_word_format(oracle, algo, fenced):
-    """The Rt64_128 family can also travel as payload lines + a separate flag word:
-    ordered by agent-scope release/acquire fences (1; 3 = payload written through),
-    or by store completion with every access at agent scope (4).  No assumption
-    about store atomicity in any of them."""
+    """The Rt64_128 family travels as the reference's messages with a flag in every
+    64 bytes (0), or as payload lines + a separate flag word: ordered by agent-scope
+    release/acquire fences (1; 3 = payload written through), or by store completion
+    with every access at agent scope (4, what the all-to-all flows take when left
+    alone).  No assumption about store atomicity in 1, 3 and 4."""
     ctx = vr.VirtualRanks(8)
     ctx.set_tuning(wire_fenced=fenced)
     for n in (64, 64 * 129, 1 << 18, 32 * 1001):
@@ -411,6 +424,7 @@ def test_embedded_flag_formats_under_repetition(ctxs, oracle, algo):
     whole every time."""
     from gpu_ipc_example_amd.binding import DeviceBuffer
     ctx = ctxs[8]
+    ctx.set_tuning(wire_fenced=0)          # the reference's embedded-flag messages for every family
     n = 8 * 8192
     ins = H.make_inputs(oracle, 8, n, 6200)
     want = H.expected(oracle, algo, ins)
@@ -424,5 +438,6 @@ def test_embedded_flag_formats_under_repetition(ctxs, oracle, algo):
             ctx.check()
             for r, b in enumerate(dst):
                 assert oracle.count_mismatch(b.download(np.uint16, n), want) == 0, (algo, it, r)
+    ctx.set_tuning(wire_fenced=-1)
     for b in src + dst:
         b.free()
