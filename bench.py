@@ -29,13 +29,15 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("cfg3", "direct"): (536914021, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
     ("cfg4", "direct"): (167799218, "direct_allreduce_bisect_8x32MiB_hbm_traffic.md"),
-    ("cfg5_32MiB", "wire"): (1551376119, "wire_allreduce_parallel_8x32MiB.md"),
-    ("cfg3", "wire"): (1562205164, "wire_allreduce_bisect_8x32MiB.md"),
+    ("cfg5_32MiB", "wire"): (1498284599, "wire_allreduce_flag_words_8x32MiB.md"),
+    ("cfg3", "wire"): (1501431833, "wire_allreduce_flag_words_8x32MiB.md"),
 }
 
 
 def measured_traffic(name, transport):
     algo = WORKLOADS[name][1]
+    if transport == "static":
+        return None
     if transport == "default":
         transport = "wire" if algo == "parallel" else "direct"
     return MEASURED_TRAFFIC_BYTES.get((name, transport), (None, None))[0]
@@ -72,6 +74,8 @@ CFG2_KERNEL_TRACE = (4.52, "direct_allreduce_small_8x1MiB_kernel_trace.md")
 
 # --transport: how the virtual ranks exchange data (0 = the protocol's default).
 TRANSPORT = 0
+# --transport static: vr_allreduce_static (wire transport through the library's fixed scratch region)
+STATIC = False
 
 
 def describe(name):
@@ -119,6 +123,9 @@ def launch(ctx, name, ins, outs):
     n, algo, ne, *_ = WORKLOADS[name]
     if algo.startswith("allgather"):
         ctx.allgather(algo, [b.ptr for b in ins], [b.ptr for b in outs], ne, transport=TRANSPORT)
+    elif STATIC:
+        # the allocation-free entry point: message passing through the library's fixed region
+        ctx.allreduce_static(algo, [b.ptr for b in ins], ne, outs=[b.ptr for b in outs] if outs else None)
     else:
         ctx.allreduce(algo, [b.ptr for b in ins], ne, outs=[b.ptr for b in outs] if outs else None,
                       transport=TRANSPORT)
@@ -171,7 +178,7 @@ def in_place_cold(binding, ctx, name, sets, host, rounds=10):
                 ctx.stream_probe(0, dst.ptr, src.ptr, ne * 2)
         timer.start(p)
         for ins, outs in sets:
-            ctx.allreduce(algo, [b.ptr for b in outs], ne, transport=TRANSPORT)
+            launch(ctx, name, outs, None)
         timer.stop(p)
     ctx.sync()
     ms = timer.elapsed_ms(rounds) / len(sets)
@@ -499,9 +506,10 @@ def main():
                          "known-size kernel that hardware-counter readings are scaled by")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"],
                     help="element type of the adds (the reference instantiates both)")
-    ap.add_argument("--transport", default="default", choices=["default", "direct", "wire"],
+    ap.add_argument("--transport", default="default", choices=["default", "direct", "wire", "static"],
                     help="direct: one pass over HBM; wire: the reference's message passing through "
-                         "scratch; default: wire for 'parallel', direct otherwise")
+                         "scratch; default: wire for 'parallel', direct otherwise; static: the "
+                         "allocation-free entry point (wire transport through the library's fixed region)")
     ap.add_argument("--inplace", action="store_true",
                     help="reference semantics: results overwrite the inputs (values saturate "
                          "after a few steps; traffic is identical)")
@@ -530,10 +538,11 @@ def main():
     import gpu_ipc_example_amd as vr
     from gpu_ipc_example_amd import binding
 
-    global DTYPE, TRANSPORT
+    global DTYPE, TRANSPORT, STATIC
     DTYPE = 1 if args.dtype == "bf16" else 0
+    STATIC = args.transport == "static"
     TRANSPORT = {"default": vr.TRANSPORT_DEFAULT, "direct": vr.TRANSPORT_DIRECT,
-                 "wire": vr.TRANSPORT_WIRE}[args.transport]
+                 "wire": vr.TRANSPORT_WIRE, "static": vr.TRANSPORT_WIRE}[args.transport]
 
     if args.sweep:
         sweep(vr, binding, args)
