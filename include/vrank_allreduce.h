@@ -93,9 +93,12 @@ typedef enum vr_algo {
  *          except VR_ALGO_PARALLEL.
  *  WIRE  : the reference's stage structure — scatter into the owner's sink,
  *          reduce, gather into every peer's sink — through the context's scratch,
- *          with a flag inside every message (or, on request, separate flag words
- *          ordered by agent-scope release/acquire fences), one persistent kernel
- *          whose workgroups are partitioned between the virtual ranks.  This is
+ *          one persistent kernel whose workgroups are partitioned between the
+ *          virtual ranks.  Receivers learn of a message from a flag: the reference's
+ *          flag inside every message (Rt64, Rt64_PCIE, and on request Rt64_128 /
+ *          Rt64_128_PCIE byte for byte), or one flag word per message beside full
+ *          payload lines, every access at agent scope (what the Rt64_128 families of
+ *          the all-to-all flows take when left alone; see "wire_fenced").  This is
  *          the form that carries over to several GPUs.  Default for
  *          VR_ALGO_PARALLEL. */
 typedef enum vr_transport {
@@ -187,10 +190,9 @@ int vr_allgather(vr_ctx *ctx, void *stream, int algo, int transport, const void 
  *   seq_no   : in/out; must be the same on every rank and only ever grow; a
  *              change of algo needs freshly zeroed sinks.
  * Same validation and error codes as vr_allreduce for this rank's pointers
- * (calcWorkSize: alignment to the protocol's message_t).  Only `parallel`, and
- * the Rt64_128 families when "wire_fenced" selects a flag-word format, move 16
- * bytes per lane whenever nelems / nranks is a multiple of 8 elements, on every
- * rank alike; input and output must then be 16-byte aligned (VR_ERR_UNALIGNED).
+ * (calcWorkSize: alignment to the protocol's message_t, 8 or 16 bytes) and
+ * nothing stricter: where a format carries 16 bytes per lane, a rank whose
+ * buffers are only 8-byte aligned moves them as two 8-byte accesses.
  * The library neither allocates nor clears anything here.  vr_ctx_check(ctx,
  * stream) reports a time-out of this context's launches; after one, the caller
  * zeroes its sinks again.
@@ -316,12 +318,17 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch
  * covers; chunks longer than this, at most 1 GiB, take several launches);
- * for the wire transport "wire_fenced" (the Rt64_128 families, instead of the
- * reference's 128 / 256-byte messages with a flag in every 64 bytes: 1 = payload
- * lines with a separate flag word ordered by agent-scope release/acquire fences,
- * 2 = self-validating 8-byte messages, 3 = as 1 with the payload stored written
- * through at agent scope, 4 = flag words with every access at agent scope, ordered
- * by store completion alone, no cache maintenance) and
+ * for the wire transport "wire_fenced" (how the Rt64_128 families, i.e. simple,
+ * bisect, parallel, simple_pcie_p, simple_ring, simple_pcie, simple_transmit,
+ * tell a receiver that a message is there: 0 = the reference's 128 / 256-byte
+ * messages with a flag in every 64 bytes; 1 = full payload lines and a separate
+ * flag word, ordered by agent-scope release / acquire fences; 2 = self-validating
+ * 8-byte messages; 3 = as 1 with the payload stored written through; 4 = flag
+ * words with every payload and flag access at agent scope (stores written
+ * through, loads never served from a stale line), the flag stored once the
+ * payload stores have completed: no cache maintenance.  Left alone (-1): 4 for
+ * the all-to-all flows ParallelTransmit / BisectPTransmit / SimpleTransmit, 0 for
+ * the ring and sequential flows) and
  * "wire_cooperative" (1 = cooperative launch; by default a plain launch: the
  * library sizes every grid within the occupancy query's bound, so it is
  * co-resident on an otherwise idle device),
