@@ -1482,7 +1482,7 @@ hipError_t launch_wire_clear_sinks(hipStream_t s, const PtrTable &scatter, const
   const size_t per_sink = (slot_bytes + flag_bytes) / 16;
   if (per_sink == 0) return hipSuccess;
   size_t bx = (per_sink + 255) / 256;
-  if (bx > 64) bx = 64;
+  if (bx > 256) bx = 256;
   hipLaunchKernelGGL(k_wire_clear_sinks, dim3((uint32_t)bx, 2u * (uint32_t)nranks), dim3(256), 0, s, scatter,
                      gather, nranks, slot_bytes, flag_off, flag_bytes);
   return hipGetLastError();

@@ -176,7 +176,10 @@ static int plan_wire(const vr_ctx *c, const AlgoInfo *a, size_t chunk_bytes, int
   if (hipError_t e = wire_blocks_per_cu(flow, fmt, vec_halves, N, kWireBlockThreads, c->dtype, &per_cu))
     return fail_hip(e, "occupancy query");
   const uint32_t resident_wpr = (uint32_t)((size_t)c->dev.cus * (size_t)per_cu / (size_t)N) * waves_per_block;
-  const uint32_t wpr_cap = k.wpr_max < resident_wpr ? k.wpr_max : resident_wpr;
+  // and within what the sinks hold for this flow (the all-to-all flows index fewer
+  // slots per wire than the ring flows the sinks are sized for)
+  const uint32_t fit = wl::wires_fitting((int)flow, N, k.layout.slots);
+  const uint32_t wpr_cap = fit < resident_wpr ? fit : resident_wpr;
   const uint32_t wpr_limit = wpr_cap / psg * psg;
   if (wpr_limit < psg) return fail(VR_ERR_INVALID, "sinks or device too small for this rank count");
   const uint32_t wire_bytes = wire_bytes_per_step(fmt, vec_halves);

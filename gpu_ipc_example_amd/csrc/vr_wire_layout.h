@@ -65,6 +65,21 @@ VR_HD size_t slots_needed(int flow, int nranks, uint32_t wpr) {
   }
 }
 
+// Largest number of wires per rank whose slot range still fits `slots` slots (the
+// inverse of slots_needed; SimpleTransmit's range does not depend on the wire
+// count).
+VR_HD uint32_t wires_fitting(int flow, int nranks, size_t slots) {
+  switch (flow) {
+    case PARALLEL: return (uint32_t)(slots / kSlotsFlat);
+    case BISECT: {
+      const size_t entries = slots / kSlotsFlat, half = (size_t)nranks / 2;
+      return entries > half ? (uint32_t)((entries - half) / 2) : 0u;
+    }
+    case SIMPLE: return slots >= (size_t)nranks * kSimplePerSection ? kSimplePerSection / 2 : 0u;
+    default: return (uint32_t)(slots / ((size_t)kSlotsRing * (size_t)nranks));
+  }
+}
+
 struct Layout {
   size_t slots;        // message slots per sink
   size_t flag_off;     // byte offset of the flag words inside a sink

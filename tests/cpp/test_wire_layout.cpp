@@ -5,6 +5,8 @@
 // No GPU, no library: plain g++.
 #include <stdio.h>
 
+#include <initializer_list>
+
 #include "vr_wire_layout.h"
 
 using namespace vr::wl;
@@ -96,6 +98,27 @@ int main() {
           }
         }
       }
+  // wires_fitting is the inverse of slots_needed: the largest wire count whose slots fit,
+  // and a walk at exactly that count stays inside the sink
+  for (int N : ranks)
+    for (size_t slots : {64u, 1000u, 1024u, 4096u, 12288u, 100000u}) {
+      Layout l = layout_for(N, 4, false);
+      l.slots = slots;
+      l.flag_off = slots * kSlotBytesMax;
+      l.sink_bytes = (l.flag_off + slots * sizeof(uint32_t) + 255) / 256 * 256;
+      for (int flow : {PARALLEL, SEQUENTIAL, RING, BISECT, ALLGATHER}) {
+        if (flow == BISECT && N < 4) continue;
+        const uint32_t fit = wires_fitting(flow, N, slots);
+        EXPECT(fit == 0 || slots_needed(flow, N, fit) <= slots);
+        EXPECT(slots_needed(flow, N, fit + 1) > slots);
+        const uint32_t psg = flow == PARALLEL ? N : flow == BISECT ? N / 2 : 1;
+        const uint32_t wpr = fit / psg * psg;
+        if (wpr >= psg && wpr <= 4096) {
+          walk(flow, N, wpr, l);
+          ++cases;
+        }
+      }
+    }
   // the fixed region of the allocation-free entry point: 8 ranks x 32 wires, no SimpleTransmit
   const Layout fixed = layout_for(8, 32, false);
   EXPECT(8 * fixed.rank_bytes + 256 <= (34u << 20));
