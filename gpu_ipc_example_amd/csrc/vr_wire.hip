@@ -1301,7 +1301,7 @@ __global__ void k_wire_clear_sinks(PtrTable scatter, PtrTable gather, int nranks
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_slots + n_flags;
        i += (size_t)gridDim.x * blockDim.x) {
     io_u32x4 *p = reinterpret_cast<io_u32x4 *>(i < n_slots ? sink + i * 16 : sink + flag_off + (i - n_slots) * 16);
-    *p = zero;
+    __builtin_nontemporal_store(zero, p);   // streamed: nothing is left dirty in L2 for the kernel's end to write back
   }
 }
 

@@ -248,8 +248,9 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
                                 "and restart from 1");
   if (wraps) seq = 1;
   if (wlch.always_clear) {
-    // only what this launch will index: its slot range and, for the flag-word
-    // formats, the flag words of those slots
+    // only what this launch will look at: the message slots of its slot range where
+    // the flag travels inside the message, the flag words of those slots where it
+    // does not (a flag-word payload is never read before its flag has been seen)
     PtrTable sc, ga;
     memset(&sc, 0, sizeof sc);
     memset(&ga, 0, sizeof ga);
@@ -258,8 +259,9 @@ static int wire_launch(vr_ctx *c, hipStream_t s, const AlgoInfo *a, const PtrTab
       ga.p[r] = k.gather[r];
     }
     const size_t slots = wl::slots_needed((int)flow, N, wpr);
-    const hipError_t e = launch_wire_clear_sinks(s, sc, ga, N, slots * wire_slot_bytes(fmt, vec_halves),
-                                                 k.layout.flag_off, wire_fmt_is_flag(fmt) ? slots * 4 : 0);
+    const bool flag_words = wire_fmt_is_flag(fmt);
+    const hipError_t e = launch_wire_clear_sinks(s, sc, ga, N, flag_words ? 0 : slots * wire_slot_bytes(fmt, vec_halves),
+                                                 k.layout.flag_off, flag_words ? slots * 4 : 0);
     if (e != hipSuccess) return fail_hip(e, "launch_wire_clear_sinks");
   } else if (wlch.hist) {
     WireHistory &h = *wlch.hist;

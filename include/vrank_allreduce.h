@@ -277,7 +277,7 @@ int vr_ipc_barrier(int rank, int world, const char *instance, int generation);
  * 32 MiB per GPU, held until the process ends) instead of scratch reserved by the
  * context.  Calls no hipMalloc / hipFree and does not synchronise.
  * Limits: at most 8 ranks, at most 256 MiB (134217728 elements) per rank, every
- * all-reduce algo except simple_transmit; 32 wires per rank.  Beyond them:
+ * all-reduce algo except simple_transmit; 32 to 128 wires per rank.  Beyond them:
  * VR_ERR_INVALID.  Every context on a GPU shares that GPU's region and each call
  * first clears the message slots it is about to use (a fill kernel on `stream`),
  * so calls that overlap in time on one GPU race: keep them on one stream or
