@@ -450,23 +450,34 @@ def latency_block(vr, binding, want_check, gpu_results, iters):
 
 
 def allgather_block(vr, binding, want_check, gpu_results):
-    """Config 4: 4 virtual ranks, all-gather of 8 MiB slices into 32 MiB outputs,
-    rotating through 4 buffer sets (640 MiB touched)."""
+    """Config 4: 4 virtual ranks, all-gather of 8 MiB slices into 32 MiB outputs.  The
+    headline figures rotate through 16 buffer sets: 512 MiB of inputs, twice the
+    256 MiB memory-side cache, so that the reads come from HBM like the writes go to
+    it (2.5 GiB touched).  With 4 sets the 128 MiB of inputs stay in that cache (the
+    streaming stores do not displace them) and only the writes reach HBM: printed as
+    `inputs_cache_resident`, not an HBM figure."""
     name = "cfg4"
     n, algo, ne, *_ = WORKLOADS[name]
-    c4, h4, s4 = setup(vr, binding, name, False, 4)
+    c4, h4, s4 = setup(vr, binding, name, False, 16)
     launch(c4, name, *s4[0])
     c4.sync()
     if want_check:
         gpu_results[name] = [b.download(np.uint16, n * ne) for b in s4[0][1]]
-    time_kernels(binding, c4, name, s4, 8)
+    time_kernels(binding, c4, name, s4, 16)
     kms, stats = kernel_sample(binding, c4, name, s4, 10)
     B = algorithmic_bytes(name)
     gb = B / (float(kms.mean()) * 1e-3) / 1e9
     out = {"workload": describe(name), "GBps": round(gb, 1), "frac_of_hbm_peak": round(gb / HBM_PEAK_GBPS, 4),
            "algorithmic_bytes_per_step": B, "traffic": measured_traffic(name, "default"),
-           "bit_exact_vs_oracle": None}
+           "buffer_sets_rotated": len(s4), "bit_exact_vs_oracle": None}
     out.update(stats)
+    time_kernels(binding, c4, name, s4[:4], 8)
+    warm, wstats = kernel_sample(binding, c4, name, s4[:4], 10)
+    wgb = B / (float(warm.mean()) * 1e-3) / 1e9
+    out["inputs_cache_resident"] = {
+        "GBps": round(wgb, 1), "kernel_us_avg": wstats["kernel_us_avg"], "buffer_sets_rotated": 4,
+        "note": "4 sets: their 128 MiB of inputs fit the 256 MiB memory-side cache, so the reads "
+                "(a fifth of the bytes) are served by it; not an HBM figure"}
     return out
 
 
@@ -570,6 +581,10 @@ def main():
     n, algo, ne, *_ = WORKLOADS[name]
     B = algorithmic_bytes(name)
     nsets = args.sets if args.sets is not None else (4 if ne * 2 <= (32 << 20) or n * ne * 2 <= (256 << 20) else 2)
+    if args.sets is None:
+        # the inputs of all sets together are at least twice the 256 MiB memory-side cache
+        # (streaming stores do not displace cached inputs, so the inputs alone must not fit it)
+        nsets = min(64, max(nsets, -(-(512 << 20) // (n * ne * 2))))
     ctx, host, sets = setup(vr, binding, name, args.inplace, nsets)
     for kv in args.tune:
         k, v = kv.split("=")

@@ -221,6 +221,7 @@ extern "C" int vr_ctx_create(int device, int nranks, vr_ctx **out) {
   c->nranks = nranks;
   c->dev.device = device;
   c->dev.cus = prop.multiProcessorCount;
+  c->dev.lds_per_cu = prop.maxSharedMemoryPerMultiProcessor;
   snprintf(c->dev.arch, sizeof c->dev.arch, "%s", prop.gcnArchName);
   c->status = status;
   *out = c;
@@ -262,6 +263,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "oneshot")) return &ctx->tune.oneshot;
   if (!strcmp(key, "segment_kib")) return &ctx->tune.segment_kib;
   if (!strcmp(key, "f16_wide")) return &ctx->tune.f16_wide;
+  if (!strcmp(key, "wgs_per_cu")) return &ctx->tune.wgs_per_cu;
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
@@ -293,6 +295,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
     if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))
       return fail(VR_ERR_INVALID, "segment_kib must be in [1, 1048576]");
+    if (!strcmp(key, "wgs_per_cu") && (value < 0 || value > 8))
+      return fail(VR_ERR_INVALID, "wgs_per_cu must be in [0,8] (0 = no cap)");
     if (!strcmp(key, "wire_ahead") && (value < 1 || value > kWireMaxSlots - 2))
       return fail(VR_ERR_INVALID, "wire_ahead must be in [1,6]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
@@ -350,6 +354,21 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     t.waves_per_cu = 32;
     t.nt_load = 0;
     t.nt_store = 2;
+    // From 64 MiB of output on: a one-trip grid (one tile per work-group).  The
+    // hardware starts work-groups in index order, so the launch sweeps every stream
+    // front to back with all CUs close together, where the work-groups of a
+    // persistent grid drift apart: 9 to 20 % faster on inputs no cache holds
+    // (4 x 8 MiB: 33.4 -> 30.5 us, 4 x 32 MiB: 126 -> 108 us, 2 x 64 MiB: 73 -> 66 us),
+    // as fast or faster when the inputs are cache-resident, slower only for
+    // launch-bound sizes.  Eight ranks write eight streams per work-group and do
+    // best with two 512-lane work-groups per CU (4 MiB per rank: 56.8 -> 52.7 us).
+    if (write_bytes >= ((size_t)64 << 20)) {
+      t.oneshot = 1;
+      if (ctx->nranks == 8 && write_bytes >= ((size_t)128 << 20)) {
+        t.block = 512;
+        t.wgs_per_cu = 2;
+      }
+    }
   } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) <= kMall) {
     // "small" family at the sizes it is meant for: every lane makes one trip;
     // results stay cacheable for the kernel that consumes them next.  (Beyond the
@@ -388,6 +407,22 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // measured 5 % (128 MiB per rank) to 9 % (256 MiB) faster than one long
       // launch; no gain at 4 or 16 ranks, a loss at 2.
       if (ctx->nranks == 8 && read_bytes / 64 >= ((size_t)16 << 20)) t.segment_bytes = (size_t)4 << 20;
+      // 2, 4 and 16 ranks: a one-trip grid (one tile per work-group, started by the
+      // hardware in index order, so the launch sweeps the buffers front to back) whose
+      // residency is capped so that about 32 KiB (64 KiB at 16 ranks) of loads per CU
+      // are in flight.  Measured on cold sets against the persistent grid: 2 ranks
+      // 0.78 -> 0.82-0.85 of peak (128 and 256 MiB per rank), 4 ranks 0.74 -> 0.79
+      // (64 MiB), 0.75 -> 0.80 (128 MiB), 0.71 -> 0.79 (256 MiB), 16 ranks 0.68-0.70
+      // -> 0.70-0.73.  Eight ranks gain nothing from it (every combination of block,
+      // vectors per lane and cap lands 1-2 % behind the persistent grid at 32 MiB per
+      // rank), so they keep it.
+      if (ctx->nranks == 2) {
+        t.oneshot = 1, t.block = 512, t.unroll = 1, t.wgs_per_cu = 2;
+      } else if (ctx->nranks == 4) {
+        t.oneshot = 1, t.block = 256, t.unroll = 1, t.wgs_per_cu = 2;
+      } else if (ctx->nranks == 16) {
+        t.oneshot = 1, t.block = 64, t.unroll = 1, t.wgs_per_cu = 4;
+      }
     }
   }
   const TuningOverrides &o = ctx->tune;
@@ -399,6 +434,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   if (o.oneshot != -1) t.oneshot = o.oneshot;
   if (o.segment_kib != -1) t.segment_bytes = (size_t)o.segment_kib << 10;
   if (o.f16_wide != -1) t.f16_wide = o.f16_wide;
+  if (o.wgs_per_cu != -1) t.wgs_per_cu = o.wgs_per_cu;
   return t;
 }
 
@@ -505,6 +541,7 @@ static int apply_user_grid(const vr_ctx *ctx, uint32_t groups, uint32_t subgroup
   t->block = (int)lanes;
   t->unroll = 1;
   t->oneshot = 0;
+  t->wgs_per_cu = 0;
   t->force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
   const uint64_t w = (uint64_t)groups * subgroups;
   *wires = w > 0xffffffffull ? 0xffffffffu : (uint32_t)w;
@@ -812,21 +849,25 @@ extern "C" int vr_time_allreduce_grouped(vr_ctx *ctx, void *stream, int algo, in
   return rc;
 }
 
-// The probes are pure streaming: streaming loads, streaming agent-scope stores,
-// four 16-byte vectors per lane in flight.  A 1:1 copy measured best with one
-// 256-lane work-group per CU, the one-way modes with 1024 lanes x 16 waves per CU.
+// The probes are pure streaming: streaming loads, streaming agent-scope stores, as
+// one-trip grids (one tile per work-group, started in index order, so the launch
+// sweeps the buffer front to back) with the residency that measured best for each:
+// a 1:1 copy with six 256-lane work-groups per CU (6.87 TB/s against 6.3 for the
+// best persistent grid), reads with two 256-lane work-groups of four vectors per
+// lane (7.3 against 6.9), writes with eight 128-lane work-groups (7.4 against 6.6).
 static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, int mode, Tuning *t) {
   if (!ctx || !dst || !src) return fail(VR_ERR_INVALID, "null argument");
   if (int rc = use_device(ctx)) return rc;
   if (bytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16)
     return fail(VR_ERR_UNALIGNED, "copy wants 16-byte granules");
   Tuning d;
-  d.block = mode == 0 ? 256 : 1024;
-  d.waves_per_cu = mode == 0 ? 4 : 16;
-  d.unroll = 4;
+  d.block = mode == 2 ? 128 : 256;
+  d.waves_per_cu = mode == 0 ? 4 : 16;     // (persistent grids only: "oneshot" = 0)
+  d.unroll = mode == 1 ? 4 : 1;
   d.nt_load = 1;
   d.nt_store = 2;
-  d.oneshot = 0;
+  d.oneshot = 1;
+  d.wgs_per_cu = mode == 0 ? 6 : mode == 1 ? 2 : 8;
   const TuningOverrides &o = ctx->tune;
   if (o.block != -1) d.block = o.block;
   if (o.waves_per_cu != -1) d.waves_per_cu = o.waves_per_cu;
@@ -834,6 +875,8 @@ static int copy_tuning(vr_ctx *ctx, void *dst, const void *src, size_t bytes, in
   if (o.nt_load != -1) d.nt_load = o.nt_load;
   if (o.nt_store != -1) d.nt_store = o.nt_store;
   if (o.segment_kib != -1) d.segment_bytes = (size_t)o.segment_kib << 10;
+  if (o.oneshot != -1) d.oneshot = o.oneshot;
+  if (o.wgs_per_cu != -1) d.wgs_per_cu = o.wgs_per_cu;
   *t = d;
   return VR_OK;
 }

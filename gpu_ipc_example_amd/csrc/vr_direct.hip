@@ -23,6 +23,10 @@
 
 #include <hip/hip_ext.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "vr_internal.h"
 
 namespace vr {
@@ -246,6 +250,32 @@ hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device
 
 // ---- host-side launch plumbing -------------------------------------------------
 
+// Residency cap of a one-trip grid.  The hardware places as many work-groups on a
+// CU as registers and LDS allow; a launch that wants at most `wgs` there asks for
+// so much dynamic LDS (never touched) that one more would not fit.  0 = no cap.
+static uint32_t lds_cap_bytes(const DeviceInfo &dev, int wgs) {
+  if (wgs <= 0 || dev.lds_per_cu == 0) return 0;
+  if (wgs > 8) wgs = 8;
+  // 15/16 of an equal share: `wgs` shares fit with room for allocation granules,
+  // wgs + 1 exceed the CU's LDS for every wgs <= 8.
+  size_t b = dev.lds_per_cu / (size_t)wgs / 16 * 15;
+  b -= b % 1024;
+  return (uint32_t)b;
+}
+
+// A kernel may ask for more than 64 KiB of dynamic LDS only after it has been told
+// so, once per kernel and device.
+static hipError_t allow_dynamic_lds(const void *kernel, int device, uint32_t bytes) {
+  if (bytes <= 48u * 1024u) return hipSuccess;
+  static std::mutex lock;
+  static std::set<std::pair<const void *, int>> done;
+  std::lock_guard<std::mutex> hold(lock);
+  if (done.count({kernel, device})) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess) done.insert({kernel, device});
+  return e;
+}
+
 // A launch addresses each chunk with 32-bit byte offsets, so longer chunks are
 // covered by several launches of at most Tuning::segment_bytes per chunk.
 static size_t segment_of(const Tuning &t) {
@@ -295,6 +325,7 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
                                      const PtrTable &in, const PtrTable &out, size_t chunk_bytes) {
   const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
   const size_t seg_max = segment_of(t);
+  const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   for (size_t off = 0; off < chunk_bytes; off += seg_max) {
     const size_t seg = chunk_bytes - off < seg_max ? chunk_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
@@ -304,10 +335,11 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
     hipEvent_t ev1 = off + seg >= chunk_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, 0, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
       else
-        hipLaunchKernelGGL(kernel, grid, block, 0, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
@@ -377,6 +409,7 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
                                      const PtrTable &in, const PtrTable &out, size_t slice_bytes) {
   const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
   const size_t seg_max = segment_of(t);
+  const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   for (size_t off = 0; off < slice_bytes; off += seg_max) {
     const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
@@ -385,10 +418,11 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
     hipEvent_t ev1 = off + seg >= slice_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, 0, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr);
       else
-        hipLaunchKernelGGL(kernel, grid, block, 0, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
@@ -428,6 +462,7 @@ static hipError_t launch_probe_segments(hipStream_t s, const DeviceInfo &dev, co
                                         char *dst, const char *src, size_t bytes) {
   const size_t tile = (size_t)t.block * 16 * UNROLL;
   const size_t seg_max = segment_of(t);
+  const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   for (size_t off = 0; off < bytes; off += seg_max) {
     const size_t seg = bytes - off < seg_max ? bytes - off : seg_max;
     size_t blocks = (seg + tile - 1) / tile;
@@ -436,8 +471,9 @@ static hipError_t launch_probe_segments(hipStream_t s, const DeviceInfo &dev, co
     if (blocks == 0) blocks = 1;
     const dim3 grid((uint32_t)blocks), block(t.block);
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
-      hipLaunchKernelGGL((k_probe<MODE, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>), grid,
-                         block, 0, s, dst + off, src + off, (uint32_t)seg);
+      auto kernel = k_probe<MODE, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
+      hipLaunchKernelGGL(kernel, grid, block, lds, s, dst + off, src + off, (uint32_t)seg);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;

@@ -314,7 +314,11 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * (persistent grid size = CUs * this / waves per block), "unroll" (16-byte
  * vectors in flight per lane and rank), "nt_load" (0 cached, 1 streaming loads),
  * "nt_store" (0 cached, 1 streaming stores, 2 streaming stores written through
- * at agent scope), "oneshot" (0/1), "f16_wide" (1 = binary16 adds computed through
+ * at agent scope), "oneshot" (1 = one-trip grid: one tile per work-group, no
+ * grid-stride loop; the hardware starts work-groups in index order, so the launch
+ * sweeps the buffers front to back), "wgs_per_cu" (0..8: at most this many
+ * work-groups of a one-trip grid share a compute unit, 0 = as many as fit),
+ * "f16_wide" (1 = binary16 adds computed through
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch
  * covers; chunks longer than this, at most 1 GiB, take several launches);

@@ -446,6 +446,70 @@ def test_every_cache_policy_gives_the_same_bits(ctxs, oracle, nt_load, nt_store)
         ctx.set_tuning(nt_load=-1, nt_store=-1, unroll=-1)
 
 
+@pytest.mark.parametrize("nranks", [2, 4, 8, 16])
+def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
+    """A one-trip grid (one tile per work-group) at every block size, vector count and
+    residency cap, on sizes whose last tile is ragged, in place and out of place, and
+    the all-gather through the same launch path."""
+    ctx = ctxs[nranks]
+    algo = "bisect" if nranks >= 4 else "simple"
+    n = nranks * 4 * 20011
+    ins = H.make_inputs(oracle, nranks, n, 9100 + nranks)
+    want = H.expected(oracle, algo, ins)
+    try:
+        for block, unroll, cap in ((64, 1, 4), (256, 1, 2), (512, 1, 2), (256, 2, 1), (1024, 4, 1), (128, 2, 8),
+                                   (256, 1, 0)):
+            ctx.set_tuning(oneshot=1, block=block, unroll=unroll, wgs_per_cu=cap)
+            what = "N=%d block=%d unroll=%d cap=%d" % (nranks, block, unroll, cap)
+            got, _ = H.run_allreduce(ctx, algo, ins)
+            H.assert_all_ranks_equal(oracle, got, want, what)
+            got, kept = H.run_allreduce(ctx, algo, ins, inplace=False, offset_bytes=8)
+            H.assert_all_ranks_equal(oracle, got, want, what + " out of place, 8-byte aligned")
+            for a, b in zip(kept, ins):
+                assert (a == b).all(), what
+        if nranks <= 8:
+            ctx.set_tuning(oneshot=1, block=512, unroll=1, wgs_per_cu=2)
+            gin = H.make_inputs(oracle, nranks, 8 * 5003, 9200 + nranks, DIST_UNIFORM, -2.0, 2.0)
+            gwant = oracle.allgather(gin)
+            for alias in (False, True):
+                got = run_allgather(ctx, "allgather_simple", gin, alias)
+                for r in range(nranks):
+                    assert (got[r] == gwant).all(), (nranks, r, alias)
+    finally:
+        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1)
+    with pytest.raises(vr.VRError):
+        ctx.set_tuning(wgs_per_cu=9)
+
+
+@pytest.mark.parametrize("nranks,algo,mib", [(2, "simple", 128), (4, "bisect", 64), (4, "simple", 64),
+                                             (16, "bisect", 16)])
+def test_streaming_shapes_of_other_rank_counts(ctxs, oracle, nranks, algo, mib):
+    """Sizes at which 2, 4 and 16 ranks stream from HBM, where the library launches its
+    one-trip grids by itself; out of place (nothing of it fits the memory-side cache)."""
+    n = (mib << 20) // 2
+    draw = 1 << 22
+    ins = [np.tile(a, n // draw) for a in H.make_inputs(oracle, nranks, draw, 9300 + nranks, DIST_NORMAL, 0.0, 0.02)]
+    want = H.expected(oracle, algo, ins)
+    got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=False)
+    assert oracle.count_mismatch(got[0], want) == 0, (nranks, algo)
+    for r in range(1, nranks):
+        assert oracle.count_mismatch(got[r], got[0]) == 0, (nranks, algo, r)
+    for a, b in zip(kept, ins):
+        assert (a == b).all()
+
+
+def test_allgather_one_trip_sizes(ctxs, oracle):
+    """All-gather shapes from 64 MiB of output on, where the library launches a one-trip
+    grid (eight ranks: with a residency cap), own slot aliased or not."""
+    for nranks, n in ((2, 1 << 24), (4, 1 << 22), (8, 1 << 21)):
+        ins = H.make_inputs(oracle, nranks, n, 9400 + nranks, DIST_UNIFORM, -2.0, 2.0)
+        want = oracle.allgather(ins)
+        for alias in (False, True):
+            got = run_allgather(ctxs[nranks], "allgather_simple", ins, alias)
+            for r in range(nranks):
+                assert (got[r] == want).all(), (nranks, r, alias)
+
+
 def test_nothing_is_written_past_the_end(ctxs, oracle):
     """The last tile of a chunk hangs over its end; the hardware bounds check of the
     buffer resource must drop those lanes (outputs carry 64 guard bytes here)."""
