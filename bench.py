@@ -512,7 +512,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["copy"],
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["copy", "read_only", "write_only"],
                     help="'copy' runs only the plain streaming copy (512 MiB per launch), the "
                          "known-size kernel that hardware-counter readings are scaled by")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"],
@@ -559,8 +559,14 @@ def main():
         sweep(vr, binding, args)
         return
 
-    if args.workload == "copy":
+    if args.workload in ("copy", "read_only", "write_only"):
+        # the streaming yardsticks alone: 512 MiB per launch, source and destination walking
+        # over eight buffers (4 GiB), median of single-launch HIP-event times
+        mode = {"copy": 0, "read_only": 1, "write_only": 2}[args.workload]
         ctx = vr.VirtualRanks(8)
+        for kv in args.tune:
+            k, v = kv.split("=")
+            ctx.set_tuning(**{k: int(v)})
         nbytes = 512 << 20
         bufs = [binding.DeviceBuffer(nbytes) for _ in range(8)]
         for b in bufs:
@@ -568,13 +574,15 @@ def main():
         timer = binding.EventTimer(args.steps)
         for k in range(args.steps):
             timer.start(k)
-            ctx.stream_probe(0, bufs[(2 * k + 1) % 8].ptr, bufs[(2 * k) % 8].ptr, nbytes)
+            ctx.stream_probe(mode, bufs[(2 * k + 1) % 8].ptr, bufs[(2 * k) % 8].ptr, nbytes)
             timer.stop(k)
         ctx.sync()
         ms = timer.elapsed_ms()
-        print(json.dumps({"metric": "plain_copy_bandwidth", "unit": "GB/s", "bytes_read": nbytes,
-                          "bytes_written": nbytes, "launches": args.steps,
-                          "value": round(2 * nbytes / (float(np.median(ms)) * 1e-3) / 1e9, 1)}))
+        moved = 2 * nbytes if mode == 0 else nbytes
+        print(json.dumps({"metric": "plain_%s_bandwidth" % args.workload, "unit": "GB/s",
+                          "bytes_read": nbytes if mode != 2 else 0, "bytes_written": nbytes if mode != 1 else 0,
+                          "launches": args.steps, "tune": args.tune,
+                          "value": round(moved / (float(np.median(ms)) * 1e-3) / 1e9, 1)}))
         return
 
     name = args.workload
