@@ -264,6 +264,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "segment_kib")) return &ctx->tune.segment_kib;
   if (!strcmp(key, "f16_wide")) return &ctx->tune.f16_wide;
   if (!strcmp(key, "wgs_per_cu")) return &ctx->tune.wgs_per_cu;
+  if (!strcmp(key, "deal")) return &ctx->tune.deal;
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
@@ -297,6 +298,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "segment_kib must be in [1, 1048576]");
     if (!strcmp(key, "wgs_per_cu") && (value < 0 || value > 8))
       return fail(VR_ERR_INVALID, "wgs_per_cu must be in [0,8] (0 = no cap)");
+    if (!strcmp(key, "deal") && (value < 0 || value > ctx->nranks || (value && ctx->nranks % value)))
+      return fail(VR_ERR_INVALID, "deal must be 0 or a divisor of the rank count");
     if (!strcmp(key, "wire_ahead") && (value < 1 || value > kWireMaxSlots - 2))
       return fail(VR_ERR_INVALID, "wire_ahead must be in [1,6]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
@@ -402,26 +405,42 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // trip's loads and its stores shortens the launch by 2.5 % at 8 ranks (0.5 %
       // at 4; it costs 1-2 % at 2 and 16 ranks and 8 % when the data is cache-resident).
       t.f16_wide = ctx->nranks == 4 || ctx->nranks == 8;
-      // Eight ranks with chunks of 16 MiB and more (128 MiB per rank and up): one
-      // launch per 4 MiB of every chunk, the shape of the 32 MiB-per-rank launch,
-      // measured 5 % (128 MiB per rank) to 9 % (256 MiB) faster than one long
-      // launch; no gain at 4 or 16 ranks, a loss at 2.
-      if (ctx->nranks == 8 && read_bytes / 64 >= ((size_t)16 << 20)) t.segment_bytes = (size_t)4 << 20;
-      // 2, 4 and 16 ranks: a one-trip grid (one tile per work-group, started by the
-      // hardware in index order, so the launch sweeps the buffers front to back) whose
-      // residency is capped so that about 32 KiB (64 KiB at 16 ranks) of loads per CU
-      // are in flight.  Measured on cold sets against the persistent grid: 2 ranks
-      // 0.78 -> 0.82-0.85 of peak (128 and 256 MiB per rank), 4 ranks 0.74 -> 0.79
-      // (64 MiB), 0.75 -> 0.80 (128 MiB), 0.71 -> 0.79 (256 MiB), 16 ranks 0.68-0.70
-      // -> 0.70-0.73.  Eight ranks gain nothing from it (every combination of block,
-      // vectors per lane and cap lands 1-2 % behind the persistent grid at 32 MiB per
-      // rank), so they keep it.
-      if (ctx->nranks == 2) {
-        t.oneshot = 1, t.block = 512, t.unroll = 1, t.wgs_per_cu = 2;
-      } else if (ctx->nranks == 4) {
-        t.oneshot = 1, t.block = 256, t.unroll = 1, t.wgs_per_cu = 2;
-      } else if (ctx->nranks == 16) {
-        t.oneshot = 1, t.block = 64, t.unroll = 1, t.wgs_per_cu = 4;
+      // One-trip grids: every work-group handles one tile and ends; the hardware starts
+      // work-groups in index order, so the launch sweeps the buffers front to back with
+      // all CUs close together, where the work-groups of a persistent grid drift apart.
+      // The residency cap keeps about 32 KiB of loads per CU in flight (64 KiB for the
+      // larger tiles), the same optimum as the persistent grid's.  `deal` says how many
+      // chunks are worked on at a time, i.e. how many XCDs share a chunk (with eight
+      // ranks: deal 8 = every XCD its own chunk, deal 2 = four XCDs per chunk, deal 1 =
+      // all CUs sweep one chunk after the other).  All of it measured on cold sets against
+      // the persistent grid (fractions of the HBM peak):
+      //   2 ranks  0.78 -> 0.82-0.85 (128, 256 MiB per rank)
+      //   4 ranks  0.74 -> 0.79 (64 MiB), 0.75-0.79 -> 0.80-0.82 (128 MiB), 0.71 -> 0.79 (256 MiB)
+      //   8 ranks  0.72-0.745 -> 0.757-0.76 (32 MiB), 0.71 -> 0.76-0.77 (40, 48 MiB), 0.73 -> 0.80
+      //            (64 MiB), 0.69 -> 0.77 (96 MiB), 0.72-0.74 -> 0.81 (128 MiB), 0.68-0.75 -> 0.775
+      //            (256 MiB), 0.69 -> 0.76 (512 MiB)
+      //   16 ranks 0.68-0.70 -> 0.72 (16 MiB), 0.72 -> 0.77 (32 MiB)
+      const size_t chunk = read_bytes / ((size_t)ctx->nranks * ctx->nranks);
+      const size_t MiB = (size_t)1 << 20;
+      t.oneshot = 1;
+      switch (ctx->nranks) {
+        case 2:
+          t.block = 512, t.unroll = 1, t.wgs_per_cu = 2;
+          break;
+        case 4:
+          t.block = 256, t.unroll = 1, t.wgs_per_cu = 2;
+          if (chunk >= 32 * MiB) t.deal = 1;
+          break;
+        case 8:
+          if (chunk < 8 * MiB) t.block = 128, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 2;
+          else if (chunk < 32 * MiB) t.block = 256, t.unroll = 2, t.wgs_per_cu = 1, t.deal = 2;
+          else if (chunk < 64 * MiB) t.block = 256, t.unroll = 2, t.wgs_per_cu = 1, t.deal = 1;
+          else t.block = 128, t.unroll = 1, t.wgs_per_cu = 2;
+          break;
+        default:   // 16
+          if (chunk < 2 * MiB) t.block = 256, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 8;
+          else t.block = 128, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 4;
+          break;
       }
     }
   }
@@ -435,6 +454,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   if (o.segment_kib != -1) t.segment_bytes = (size_t)o.segment_kib << 10;
   if (o.f16_wide != -1) t.f16_wide = o.f16_wide;
   if (o.wgs_per_cu != -1) t.wgs_per_cu = o.wgs_per_cu;
+  if (o.deal != -1) t.deal = o.deal;
   return t;
 }
 
@@ -542,6 +562,7 @@ static int apply_user_grid(const vr_ctx *ctx, uint32_t groups, uint32_t subgroup
   t->unroll = 1;
   t->oneshot = 0;
   t->wgs_per_cu = 0;
+  t->deal = 0;
   t->force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
   const uint64_t w = (uint64_t)groups * subgroups;
   *wires = w > 0xffffffffull ? 0xffffffffu : (uint32_t)w;

@@ -136,9 +136,15 @@ template <int N, int ORDER, int DT, typename V, int UNROLL, int LD_AUX, int ST_A
 __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable out,
                                                            size_t chunk_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank) {
-  const int owner = owner_of_group<N, ORDER>((int)(blockIdx.x % N));
-  const uint32_t jblock = blockIdx.x / N;
+                                                           uint32_t blocks_per_rank, uint32_t deal) {
+  // `deal` chunks are worked on at a time: the first deal * blocks_per_rank work-groups
+  // belong to the first `deal` owners, round robin, and so on.  deal = N: work-group b
+  // serves owner b % N throughout (with 8 ranks every XCD its own chunk); deal = 1: all
+  // work-groups, and with them all XCDs, sweep one chunk after the other.
+  const uint32_t per = deal * blocks_per_rank;
+  const uint32_t part = blockIdx.x / per, rem = blockIdx.x % per;
+  const int owner = owner_of_group<N, ORDER>((int)(part * deal + rem % deal));
+  const uint32_t jblock = rem / deal;
   const size_t base = (size_t)chunk_of_owner<N, ORDER>(owner) * chunk_pitch + seg_off;
 
   __amdgpu_buffer_rsrc_t src[N], dst[N];
@@ -326,6 +332,8 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
   const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
+  // chunks dealt at a time: a divisor of N, N itself unless the launch says otherwise
+  uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
   for (size_t off = 0; off < chunk_bytes; off += seg_max) {
     const size_t seg = chunk_bytes - off < seg_max ? chunk_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
@@ -337,9 +345,9 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
       auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;

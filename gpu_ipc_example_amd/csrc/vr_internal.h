@@ -42,6 +42,8 @@ struct Tuning {
   int oneshot = 0;        // 1: grid covers the whole buffer, no grid-stride loop
   int f16_wide = 0;       // 1: binary16 adds through binary32 (same bits, longer ALU section)
   uint32_t force_blocks_per_rank = 0;  // non-zero: use exactly this many blocks per rank
+  int deal = 0;           // chunks the work-groups of an all-reduce work on at a time (a divisor of the rank
+                          // count; 0 = all of them: work-group b serves owner b % N throughout)
   int wgs_per_cu = 0;     // non-zero: at most this many work-groups of the launch share a CU (the launch
                           // asks for dynamic LDS it never touches, so that no more fit); for one-trip grids,
                           // whose residency the grid size does not bound

@@ -318,6 +318,9 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * grid-stride loop; the hardware starts work-groups in index order, so the launch
  * sweeps the buffers front to back), "wgs_per_cu" (0..8: at most this many
  * work-groups of a one-trip grid share a compute unit, 0 = as many as fit),
+ * "deal" (chunks the work-groups of an all-reduce work on at a time: a divisor
+ * of the rank count, 0 = all of them, i.e. work-group b serves owner b % N
+ * throughout; 1 = all compute units sweep one chunk after the other),
  * "f16_wide" (1 = binary16 adds computed through
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch

@@ -457,10 +457,10 @@ def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
     ins = H.make_inputs(oracle, nranks, n, 9100 + nranks)
     want = H.expected(oracle, algo, ins)
     try:
-        for block, unroll, cap in ((64, 1, 4), (256, 1, 2), (512, 1, 2), (256, 2, 1), (1024, 4, 1), (128, 2, 8),
-                                   (256, 1, 0)):
-            ctx.set_tuning(oneshot=1, block=block, unroll=unroll, wgs_per_cu=cap)
-            what = "N=%d block=%d unroll=%d cap=%d" % (nranks, block, unroll, cap)
+        for block, unroll, cap, deal in ((64, 1, 4, 1), (256, 1, 2, 2), (512, 1, 2, nranks), (256, 2, 1, 1),
+                                         (1024, 4, 1, 2), (128, 2, 8, nranks // 2), (256, 1, 0, 0)):
+            ctx.set_tuning(oneshot=1, block=block, unroll=unroll, wgs_per_cu=cap, deal=deal)
+            what = "N=%d block=%d unroll=%d cap=%d deal=%d" % (nranks, block, unroll, cap, deal)
             got, _ = H.run_allreduce(ctx, algo, ins)
             H.assert_all_ranks_equal(oracle, got, want, what)
             got, kept = H.run_allreduce(ctx, algo, ins, inplace=False, offset_bytes=8)
@@ -476,18 +476,29 @@ def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
                 for r in range(nranks):
                     assert (got[r] == gwant).all(), (nranks, r, alias)
     finally:
-        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1)
+        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1, deal=-1)
+    # chunk dealing of the persistent grid (which XCDs share a chunk)
+    try:
+        for deal in (1, 2, nranks):
+            ctx.set_tuning(oneshot=0, deal=deal)
+            got, _ = H.run_allreduce(ctx, algo, ins)
+            H.assert_all_ranks_equal(oracle, got, want, "persistent grid, deal %d" % deal)
+    finally:
+        ctx.set_tuning(oneshot=-1, deal=-1)
     with pytest.raises(vr.VRError):
         ctx.set_tuning(wgs_per_cu=9)
+    with pytest.raises(vr.VRError):
+        ctx.set_tuning(deal=3)
 
 
 @pytest.mark.parametrize("nranks,algo,mib", [(2, "simple", 128), (4, "bisect", 64), (4, "simple", 64),
-                                             (16, "bisect", 16)])
+                                             (4, "bisect", 128), (16, "bisect", 16), (16, "bisect", 32),
+                                             (8, "simple", 40), (8, "bisect", 64), (8, "simple", 96)])
 def test_streaming_shapes_of_other_rank_counts(ctxs, oracle, nranks, algo, mib):
     """Sizes at which 2, 4 and 16 ranks stream from HBM, where the library launches its
     one-trip grids by itself; out of place (nothing of it fits the memory-side cache)."""
     n = (mib << 20) // 2
-    draw = 1 << 22
+    draw = 1 << 20
     ins = [np.tile(a, n // draw) for a in H.make_inputs(oracle, nranks, draw, 9300 + nranks, DIST_NORMAL, 0.0, 0.02)]
     want = H.expected(oracle, algo, ins)
     got, kept = H.run_allreduce(ctxs[nranks], algo, ins, inplace=False)

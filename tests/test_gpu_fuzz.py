@@ -1,6 +1,6 @@
 """Randomised parity sweep: random world size, protocol, transport, element
 count, alignment, in/out-of-place choice and launch knobs (cache policy, unroll,
-residency, block size, one-trip grids and their residency cap, segment length, scatter run-ahead, wire format variant, streaming I/O),
+residency, block size, one-trip grids, their residency cap and chunk dealing, segment length, scatter run-ahead, wire format variant, streaming I/O),
 each checked bit for bit against
 the oracle.  Seeds are fixed, so a failure names a reproducible case."""
 import random
@@ -42,7 +42,8 @@ def test_random_cases(oracle, seed):
         # (drawn from a generator of their own, so that the cases above stay what they were)
         rng2 = random.Random(77_000 * seed + case)
         knobs.update(oneshot=rng2.choice((-1, -1, 0, 1)), wgs_per_cu=rng2.choice((-1, 0, 1, 2, 4, 8)),
-                     block=rng2.choice((-1, -1, 64, 256, 512, 1024)))
+                     block=rng2.choice((-1, -1, 64, 256, 512, 1024)),
+                     deal=rng2.choice((-1, -1, 0, 1, 2, nranks)))
         ctxs[nranks].set_tuning(**knobs)
         ins = H.make_inputs(oracle, nranks, n, 10_000 * seed + 37 * case,
                             p1=rng.choice((0.02, 1.0, 30.0, 3000.0)))
