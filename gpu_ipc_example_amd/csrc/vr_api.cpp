@@ -296,8 +296,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "nt_store must be 0 (cached), 1 (streaming), 2 (streaming, written through at agent scope) or -1 (automatic)");
     if (!strcmp(key, "segment_kib") && (value < 1 || value > (1 << 20)))
       return fail(VR_ERR_INVALID, "segment_kib must be in [1, 1048576]");
-    if (!strcmp(key, "wgs_per_cu") && (value < 0 || value > 8))
-      return fail(VR_ERR_INVALID, "wgs_per_cu must be in [0,8] (0 = no cap)");
+    if (!strcmp(key, "wgs_per_cu") && (value < 0 || value > 12))
+      return fail(VR_ERR_INVALID, "wgs_per_cu must be in [0,12] (0 = no cap)");
     if (!strcmp(key, "deal") && (value < 0 || value > ctx->nranks || (value && ctx->nranks % value)))
       return fail(VR_ERR_INVALID, "deal must be 0 or a divisor of the rank count");
     if (!strcmp(key, "wire_ahead") && (value < 1 || value > kWireMaxSlots - 2))
@@ -408,38 +408,38 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // One-trip grids: every work-group handles one tile and ends; the hardware starts
       // work-groups in index order, so the launch sweeps the buffers front to back with
       // all CUs close together, where the work-groups of a persistent grid drift apart.
-      // The residency cap keeps about 32 KiB of loads per CU in flight (64 KiB for the
-      // larger tiles), the same optimum as the persistent grid's.  `deal` says how many
-      // chunks are worked on at a time, i.e. how many XCDs share a chunk (with eight
-      // ranks: deal 8 = every XCD its own chunk, deal 2 = four XCDs per chunk, deal 1 =
-      // all CUs sweep one chunk after the other).  All of it measured on cold sets against
-      // the persistent grid (fractions of the HBM peak):
+      // Small work-groups (one wave) with a residency cap of 4 to 10 per CU keep 32 to
+      // 64 KiB of loads per CU in flight.  `deal` says how many chunks are worked on at a
+      // time, i.e. how many XCDs share a chunk (with eight ranks: deal 8 = every XCD its
+      // own chunk, deal 1 = all CUs sweep one chunk after the other, which is what lets
+      // the write side of HBM run: eight write streams that all XCDs fill together take
+      // 40.6 us for 256 MiB, the same streams filled one XCD per chunk 43-46 us).
+      // Measured on cold sets against the persistent grid it replaces (fractions of the
+      // HBM peak, HIP events):
       //   2 ranks  0.78 -> 0.82-0.85 (128, 256 MiB per rank)
-      //   4 ranks  0.74 -> 0.79 (64 MiB), 0.75-0.79 -> 0.80-0.82 (128 MiB), 0.71 -> 0.79 (256 MiB)
-      //   8 ranks  0.72-0.745 -> 0.757-0.76 (32 MiB), 0.71 -> 0.76-0.77 (40, 48 MiB), 0.73 -> 0.80
-      //            (64 MiB), 0.69 -> 0.77 (96 MiB), 0.72-0.74 -> 0.81 (128 MiB), 0.68-0.75 -> 0.775
-      //            (256 MiB), 0.69 -> 0.76 (512 MiB)
-      //   16 ranks 0.68-0.70 -> 0.72 (16 MiB), 0.72 -> 0.77 (32 MiB)
+      //   4 ranks  0.74-0.78 -> 0.82 (64 MiB), 0.75-0.79 -> 0.83 (128 MiB), 0.71 -> 0.82 (256 MiB)
+      //   8 ranks  0.72-0.75 -> 0.805 (32 MiB), 0.71 -> 0.79 (40, 48 MiB), 0.73 -> 0.82 (64 MiB),
+      //            0.69 -> 0.81 (96 MiB), 0.72-0.74 -> 0.82 (128 MiB), 0.68-0.75 -> 0.81 (256 MiB),
+      //            0.69 -> 0.78 (512 MiB)
+      //   16 ranks 0.68-0.70 -> 0.75 (16 MiB), 0.72 -> 0.78 (32 MiB), 0.71 -> 0.79 (64 MiB)
       const size_t chunk = read_bytes / ((size_t)ctx->nranks * ctx->nranks);
       const size_t MiB = (size_t)1 << 20;
       t.oneshot = 1;
+      t.unroll = 1;
       switch (ctx->nranks) {
         case 2:
-          t.block = 512, t.unroll = 1, t.wgs_per_cu = 2;
+          t.block = 512, t.wgs_per_cu = 2;
           break;
         case 4:
-          t.block = 256, t.unroll = 1, t.wgs_per_cu = 2;
-          if (chunk >= 32 * MiB) t.deal = 1;
+          if (chunk < 64 * MiB) t.block = 64, t.wgs_per_cu = 10, t.deal = chunk < 32 * MiB ? 2 : 1;
+          else t.block = 256, t.wgs_per_cu = 2, t.deal = 1;
           break;
         case 8:
-          if (chunk < 8 * MiB) t.block = 128, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 2;
-          else if (chunk < 32 * MiB) t.block = 256, t.unroll = 2, t.wgs_per_cu = 1, t.deal = 2;
-          else if (chunk < 64 * MiB) t.block = 256, t.unroll = 2, t.wgs_per_cu = 1, t.deal = 1;
-          else t.block = 128, t.unroll = 1, t.wgs_per_cu = 2;
+          t.block = 64, t.deal = 1;
+          t.wgs_per_cu = (chunk >= 16 * MiB && chunk <= 32 * MiB) ? 6 : 5;
           break;
         default:   // 16
-          if (chunk < 2 * MiB) t.block = 256, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 8;
-          else t.block = 128, t.unroll = 1, t.wgs_per_cu = 2, t.deal = 4;
+          t.block = 64, t.wgs_per_cu = 4, t.deal = chunk < 2 * MiB ? 2 : 1;
           break;
       }
     }

@@ -261,9 +261,9 @@ hipError_t launch_xcc_probe(hipStream_t s, uint32_t blocks, uint32_t *out_device
 // so much dynamic LDS (never touched) that one more would not fit.  0 = no cap.
 static uint32_t lds_cap_bytes(const DeviceInfo &dev, int wgs) {
   if (wgs <= 0 || dev.lds_per_cu == 0) return 0;
-  if (wgs > 8) wgs = 8;
+  if (wgs > 12) wgs = 12;
   // 15/16 of an equal share: `wgs` shares fit with room for allocation granules,
-  // wgs + 1 exceed the CU's LDS for every wgs <= 8.
+  // wgs + 1 exceed the CU's LDS for every wgs <= 12.
   size_t b = dev.lds_per_cu / (size_t)wgs / 16 * 15;
   b -= b % 1024;
   return (uint32_t)b;

@@ -316,7 +316,7 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * "nt_store" (0 cached, 1 streaming stores, 2 streaming stores written through
  * at agent scope), "oneshot" (1 = one-trip grid: one tile per work-group, no
  * grid-stride loop; the hardware starts work-groups in index order, so the launch
- * sweeps the buffers front to back), "wgs_per_cu" (0..8: at most this many
+ * sweeps the buffers front to back), "wgs_per_cu" (0..12: at most this many
  * work-groups of a one-trip grid share a compute unit, 0 = as many as fit),
  * "deal" (chunks the work-groups of an all-reduce work on at a time: a divisor
  * of the rank count, 0 = all of them, i.e. work-group b serves owner b % N

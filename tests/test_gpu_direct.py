@@ -486,7 +486,7 @@ def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
     finally:
         ctx.set_tuning(oneshot=-1, deal=-1)
     with pytest.raises(vr.VRError):
-        ctx.set_tuning(wgs_per_cu=9)
+        ctx.set_tuning(wgs_per_cu=13)
     with pytest.raises(vr.VRError):
         ctx.set_tuning(deal=3)
 
