@@ -372,7 +372,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
         t.wgs_per_cu = 2;
       }
     }
-  } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) <= kMall) {
+  } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) < kMall) {
     // "small" family at the sizes it is meant for: every lane makes one trip;
     // results stay cacheable for the kernel that consumes them next.  (Beyond the
     // cache it streams like the other protocols.)
@@ -387,7 +387,11 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     // out of place, and 3 % faster when an in-place 256 MiB set turns out not to be
     // resident after all.
     const int cached_waves = ctx->nranks == 8 ? 4 : 8;
-    if (footprint <= kMall) {            // everything can live in the memory-side cache
+    // (A footprint of exactly the cache's size counts as streaming: nothing else may have
+    // touched memory for it to be resident, and the streaming launch takes 82 us on eight
+    // 32 MiB buffers in place whether they are resident or not, where the cached policy
+    // takes 77 us if they are and 93-104 us if they are not.)
+    if (footprint < kMall) {             // everything can live in the memory-side cache
       t.waves_per_cu = cached_waves;
       t.nt_load = 0;
       t.nt_store = 1;
