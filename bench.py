@@ -498,8 +498,9 @@ def cfg5_block(vr, binding):
     out = {"sizes_bytes_per_rank": sizes,
            "parallel": sweep_rows(vr, binding, ctx, bufs, host, "parallel", vr.TRANSPORT_WIRE, sizes, iters_for),
            "direct_simple": sweep_rows(vr, binding, ctx, bufs, host, "simple", vr.TRANSPORT_DIRECT, sizes, iters_for),
-           "note": "8 virtual ranks, N(0,1), in place on one buffer set (1 MiB and 32 MiB per rank are "
-                   "served by the caches, 256 MiB per rank streams from HBM); median of single-launch "
+           "note": "8 virtual ranks, N(0,1), in place on one buffer set (1 MiB per rank is served by the "
+                   "caches; 32 MiB per rank, a footprint of exactly the memory-side cache's size, and 256 MiB "
+                   "per rank are launched as streaming); median of single-launch "
                    "HIP-event times; the full 17-point curves: bench.py --sweep"}
     for b in bufs:
         b.free()
