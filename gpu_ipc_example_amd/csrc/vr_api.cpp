@@ -363,14 +363,14 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     // persistent grid drift apart: 9 to 20 % faster on inputs no cache holds
     // (4 x 8 MiB: 33.4 -> 30.5 us, 4 x 32 MiB: 126 -> 108 us, 2 x 64 MiB: 73 -> 66 us),
     // as fast or faster when the inputs are cache-resident, slower only for
-    // launch-bound sizes.  Eight ranks write eight streams per work-group and do
-    // best with two 512-lane work-groups per CU (4 MiB per rank: 56.8 -> 52.7 us).
+    // launch-bound sizes.  From four ranks on, two sources are worked on at a time
+    // (half of the XCDs share a source's slice) rather than every XCD staying with one
+    // source: another 2-5 % (4 x 8 MiB 30.0 us, 8 x 4 MiB 53.5 -> 51.4 us); the largest
+    // eight-rank shapes do best with four work-groups per CU (8 x 16 MiB: 193.6 us).
     if (write_bytes >= ((size_t)64 << 20)) {
       t.oneshot = 1;
-      if (ctx->nranks == 8 && write_bytes >= ((size_t)128 << 20)) {
-        t.block = 512;
-        t.wgs_per_cu = 2;
-      }
+      if (ctx->nranks >= 4) t.deal = 2;
+      if (ctx->nranks == 8 && write_bytes >= ((size_t)512 << 20)) t.wgs_per_cu = 4;
     }
   } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) < kMall) {
     // "small" family at the sizes it is meant for: every lane makes one trip;

@@ -184,9 +184,14 @@ template <int N, typename V, int UNROLL, int LD_AUX, int ST_AUX>
 __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable out,
                                                            size_t slice_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank) {
-  const int p = blockIdx.x % N;
-  const uint32_t jblock = blockIdx.x / N;
+                                                           uint32_t blocks_per_rank, uint32_t deal) {
+  // `deal` source slices are worked on at a time (see k_direct_allreduce): deal = N gives
+  // work-group b to source b % N throughout, deal = 1 lets all work-groups sweep one
+  // source's slice after the other.
+  const uint32_t per = deal * blocks_per_rank;
+  const uint32_t part = blockIdx.x / per, rem = blockIdx.x % per;
+  const int p = (int)(part * deal + rem % deal);
+  const uint32_t jblock = rem / deal;
   const char *src_ptr = static_cast<const char *>(in.p[p]) + seg_off;
   const __amdgpu_buffer_rsrc_t src = make_rsrc(src_ptr, seg_bytes);
   __amdgpu_buffer_rsrc_t dst[N];
@@ -418,6 +423,7 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
   const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
+  const uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
   for (size_t off = 0; off < slice_bytes; off += seg_max) {
     const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
@@ -428,9 +434,9 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
       auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
