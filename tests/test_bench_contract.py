@@ -50,7 +50,7 @@ def test_default_line_carries_the_fixed_sample_and_the_other_configurations():
     for key in ("kernel_us_min", "kernel_us_p50", "kernel_us_p99", "n_pairs", "in_place_cold",
                 "cfg4_allgather", "cfg5_sweep_points", "latency_1MiB_per_rank", "host_call_us",
                 "back_to_back_us_per_launch", "kernel_trace_p50_us", "same_buffers_cache_warm",
-                "hbm_ceilings", "cpu_baseline", "roofline"):
+                "hbm_ceilings", "cpu_baseline", "roofline", "inputs_cache_resident", "buffer_sets_rotated"):
         assert '"%s"' % key in src, key
     us, fname = bench.CFG2_KERNEL_TRACE
     text = open(os.path.join(ROOT, "profiles", fname)).read()
@@ -64,3 +64,12 @@ def test_tiled_inputs_are_the_same_on_both_sides():
     import bench
     src = open(os.path.join(ROOT, "bench.py")).read()
     assert src.count("min(ne, 1 << 24)") == 2
+
+
+def test_rotating_sets_keep_the_inputs_out_of_the_memory_side_cache():
+    """Streaming stores do not displace cached inputs, so a workload's inputs alone, over all the sets
+    its steps rotate through, must exceed the 256 MiB cache: config 4's block rotates 16 sets
+    (512 MiB of inputs) and the default set count of every workload is raised alike."""
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    assert 'setup(vr, binding, name, False, 16)' in src
+    assert "(512 << 20) // (n * ne * 2)" in src
