@@ -1089,7 +1089,8 @@ extern "C" int vr_device_name(int device, char *buf, size_t buflen) {
   if (!buf || !buflen) return fail(VR_ERR_INVALID, "null argument");
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, device));
-  snprintf(buf, buflen, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+  snprintf(buf, buflen, "%s (%s, %d CUs, %zu KiB LDS per CU)", prop.name, prop.gcnArchName, prop.multiProcessorCount,
+           (size_t)prop.maxSharedMemoryPerMultiProcessor >> 10);
   return VR_OK;
 }
 
