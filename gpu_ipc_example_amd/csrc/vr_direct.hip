@@ -5,10 +5,16 @@
 // flat transmits, parallel_transmit.hpp:104; chunk (R&1)*N/2 + R/2 for bisect,
 // bisect_transmit.hpp:439-444,462-469): they read that chunk from every rank's
 // input (the "scatter", pulled instead of pushed), add in the reference's order,
-// and write the result into every rank's output (the "gather").  With block b
-// serving rank b % N and HIP handing consecutive blocks to consecutive XCDs, an
-// 8-rank launch gives each XCD exactly one rank's chunk: no two L2s ever touch
-// the same line.
+// and write the result into every rank's output (the "gather").
+//
+// Two grids.  Cache-resident data: a persistent grid with a grid-stride loop, block b
+// serving rank b % N; HIP hands consecutive blocks to consecutive XCDs, so an 8-rank
+// launch gives each XCD exactly one rank's chunk and no two L2s touch the same line.
+// Data streamed from HBM: a one-trip grid, one tile per work-group; the hardware
+// starts work-groups in index order, so the launch sweeps the buffers front to back,
+// its residency capped through dynamic LDS that is never touched, and the chunks dealt
+// to the work-groups one (or a few) at a time, so that all XCDs fill the same region
+// of every output together, which is how HBM's write side runs best.
 //
 // Per 16-byte column a lane issues N independent dwordx4 loads, N-1 packed
 // binary16 adds per half2, and N dwordx4 stores; nothing is staged in LDS
@@ -276,13 +282,14 @@ static uint32_t lds_cap_bytes(const DeviceInfo &dev, int wgs) {
 
 // A kernel may ask for more than 64 KiB of dynamic LDS only after it has been told
 // so, once per kernel and device.
-static hipError_t allow_dynamic_lds(const void *kernel, int device, uint32_t bytes) {
+static hipError_t allow_dynamic_lds(const void *kernel, const DeviceInfo &dev, uint32_t bytes) {
+  const int device = dev.device;
   if (bytes <= 48u * 1024u) return hipSuccess;
   static std::mutex lock;
   static std::set<std::pair<const void *, int>> done;
   std::lock_guard<std::mutex> hold(lock);
   if (done.count({kernel, device})) return hipSuccess;
-  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dev.lds_per_cu);
   if (e == hipSuccess) done.insert({kernel, device});
   return e;
 }
@@ -348,7 +355,7 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
     hipEvent_t ev1 = off + seg >= chunk_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
-      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
         hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal);
       else
@@ -432,7 +439,7 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
     hipEvent_t ev1 = off + seg >= slice_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
-      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
         hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal);
       else
@@ -486,7 +493,7 @@ static hipError_t launch_probe_segments(hipStream_t s, const DeviceInfo &dev, co
     const dim3 grid((uint32_t)blocks), block(t.block);
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_probe<MODE, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
-      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev.device, lds); a != hipSuccess) return a;
+      if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       hipLaunchKernelGGL(kernel, grid, block, lds, s, dst + off, src + off, (uint32_t)seg);
       return hipGetLastError();
     });

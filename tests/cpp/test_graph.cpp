@@ -161,6 +161,58 @@ int main() {
     (void)hipGraphDestroy(g3);
   }
 
+  // A streaming launch under capture: two ranks of 80 MiB, out of place, run as a one-trip
+  // grid whose residency is capped with 75 KiB of dynamic LDS per work-group.  This is the
+  // first launch of that kernel in the process, so the kernel's dynamic-LDS allowance is
+  // raised while the stream is capturing.  Three replays against the oracle.
+  {
+    const size_t n2 = 41943040;
+    vr_ctx *c2;
+    VRCK(vr_ctx_create(0, 2, &c2));
+    int simple_id = -1;
+    VRCK(vr_algo_from_string("simple", &simple_id));
+    std::vector<std::vector<uint16_t>> h2(2, std::vector<uint16_t>(n2));
+    void *i2[2], *o2[2];
+    const uint16_t *hp2[2];
+    for (int r = 0; r < 2; ++r) {
+      vro_generate(h2[r].data(), n2, 900 + r, VRO_DIST_NORMAL, 0.0, 0.02);
+      hp2[r] = h2[r].data();
+      HIPCK(hipMalloc(&i2[r], n2 * 2));
+      HIPCK(hipMalloc(&o2[r], n2 * 2));
+      HIPCK(hipMemcpy(i2[r], h2[r].data(), n2 * 2, hipMemcpyHostToDevice));
+    }
+    std::vector<uint16_t> want2(n2), got2(n2);
+    vro_allreduce_rotated(want2.data(), hp2, 2, n2);
+    hipGraph_t g4;
+    hipGraphExec_t e4;
+    uint32_t seq2 = 1;
+    HIPCK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    VRCK(vr_allreduce(c2, stream, simple_id, VR_TRANSPORT_DIRECT, i2, o2, n2, &seq2));
+    HIPCK(hipStreamEndCapture(stream, &g4));
+    HIPCK(hipGraphInstantiate(&e4, g4, nullptr, nullptr, 0));
+    for (int replay = 0; replay < 3; ++replay) {
+      for (int r = 0; r < 2; ++r) HIPCK(hipMemsetAsync(o2[r], 0x77, n2 * 2, stream));
+      HIPCK(hipStreamSynchronize(stream));
+      HIPCK(hipGraphLaunch(e4, stream));
+      HIPCK(hipStreamSynchronize(stream));
+      for (int r = 0; r < 2; ++r) {
+        HIPCK(hipMemcpy(got2.data(), o2[r], n2 * 2, hipMemcpyDeviceToHost));
+        const size_t bad = vro_count_mismatch(got2.data(), want2.data(), n2);
+        if (bad) {
+          printf("streaming replay %d rank %d: %zu mismatches\n", replay, r, bad);
+          ++failures;
+        }
+      }
+    }
+    (void)hipGraphExecDestroy(e4);
+    (void)hipGraphDestroy(g4);
+    for (int r = 0; r < 2; ++r) {
+      (void)hipFree(i2[r]);
+      (void)hipFree(o2[r]);
+    }
+    vr_ctx_destroy(c2);
+  }
+
   (void)hipGraphExecDestroy(exec);
   (void)hipGraphDestroy(graph);
   for (int r = 0; r < N; ++r) {
