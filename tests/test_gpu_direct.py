@@ -467,8 +467,13 @@ def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
             H.assert_all_ranks_equal(oracle, got, want, what + " out of place, 8-byte aligned")
             for a, b in zip(kept, ins):
                 assert (a == b).all(), what
+        # chunks longer than a launch's segment: several one-trip launches per all-reduce, the last one ragged
+        ctx.set_tuning(oneshot=1, block=64, unroll=1, wgs_per_cu=5, deal=1, segment_kib=16)
+        got, _ = H.run_allreduce(ctx, algo, ins)
+        H.assert_all_ranks_equal(oracle, got, want, "N=%d one-trip in 16 KiB segments" % nranks)
+        ctx.set_tuning(segment_kib=-1)
         if nranks <= 8:
-            ctx.set_tuning(oneshot=1, block=512, unroll=1, wgs_per_cu=2)
+            ctx.set_tuning(oneshot=1, block=512, unroll=1, wgs_per_cu=2, deal=2)
             gin = H.make_inputs(oracle, nranks, 8 * 5003, 9200 + nranks, DIST_UNIFORM, -2.0, 2.0)
             gwant = oracle.allgather(gin)
             for alias in (False, True):
@@ -476,7 +481,7 @@ def test_one_trip_grids_with_a_residency_cap(ctxs, oracle, nranks):
                 for r in range(nranks):
                     assert (got[r] == gwant).all(), (nranks, r, alias)
     finally:
-        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1, deal=-1)
+        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1, deal=-1, segment_kib=-1)
     # chunk dealing of the persistent grid (which XCDs share a chunk)
     try:
         for deal in (1, 2, nranks):
