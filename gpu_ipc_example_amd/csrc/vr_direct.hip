@@ -280,8 +280,8 @@ static uint32_t lds_cap_bytes(const DeviceInfo &dev, int wgs) {
   return (uint32_t)b;
 }
 
-// A kernel may ask for more than 64 KiB of dynamic LDS only after it has been told
-// so, once per kernel and device.
+// A kernel may ask for more than 48 KiB of dynamic LDS only after its limit has been
+// raised, once per kernel and device.
 static hipError_t allow_dynamic_lds(const void *kernel, const DeviceInfo &dev, uint32_t bytes) {
   const int device = dev.device;
   if (bytes <= 48u * 1024u) return hipSuccess;
