@@ -395,6 +395,13 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       t.waves_per_cu = cached_waves;
       t.nt_load = 0;
       t.nt_store = 1;
+      // Out of place with inputs about the size of the L2s together (8 x 4 MiB): results
+      // that allocate there push out inputs still to be read; written through, they leave
+      // them alone (32 MiB of inputs: 10.1 -> 8.7 us at 8 ranks, 10.3 -> 8.6 at 4, 11.4 -> 9.1
+      // at 2; 40 MiB: 1-7 % faster).  Not below: those launches are latency-bound and
+      // written-through stores end them 0.3-0.5 us later; no difference beyond.
+      const size_t MiB = (size_t)1 << 20;
+      if (!in_place && read_bytes > 24 * MiB && read_bytes <= 40 * MiB) t.nt_store = 2;
     } else if (read_bytes <= kMall / 2) {  // inputs may still be resident; stream the results past them
       t.waves_per_cu = cached_waves;
       t.nt_load = 0;
