@@ -96,3 +96,30 @@ def test_dtype_switch_on_one_context(oracle):
     with pytest.raises(vr.VRError):
         ctx.set_dtype(7)
     ctx.close()
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8, 16])
+def test_bf16_one_trip_grids_and_streaming_sizes(oracle, nranks):
+    """The bfloat16 instantiation under the launches streaming sizes get: forced one-trip grids
+    (residency cap, chunk dealing) on ragged sizes, then the library's own choice at 256 MiB of
+    inputs, where it streams."""
+    ctx = vr.VirtualRanks(nranks)
+    ctx.set_dtype(binding.DTYPE_BF16)
+    algos = ("bisect",) if nranks == 16 else ("simple",) if nranks == 2 else ("simple", "bisect")
+    n = 8 * nranks * 4099
+    ins = [oracle.generate_dt(BF16, n, 700 + r, DIST_NORMAL, 0.0, 1.0) for r in range(nranks)]
+    for algo in algos:
+        want = oracle.order_dt(BF16, 2 if algo == "bisect" else 1, ins)
+        for block, cap, deal in ((64, 5, 1), (256, 2, 2), (128, 0, nranks)):
+            ctx.set_tuning(oneshot=1, block=block, unroll=1, wgs_per_cu=cap, deal=deal)
+            for inplace in (True, False):
+                for r, g in enumerate(run(ctx, algo, ins, vr.TRANSPORT_DIRECT, inplace)):
+                    assert oracle.count_mismatch_dt(BF16, g, want) == 0, (algo, block, cap, deal, inplace, r)
+        ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1, deal=-1)
+    n = (256 << 20) // 2 // nranks
+    ins = [oracle.generate_dt(BF16, n, 900 + r, DIST_NORMAL, 0.0, 0.02) for r in range(nranks)]
+    algo = algos[-1]
+    want = oracle.order_dt(BF16, 2 if algo == "bisect" else 1, ins)
+    for r, g in enumerate(run(ctx, algo, ins, vr.TRANSPORT_DIRECT, inplace=False)):
+        assert oracle.count_mismatch_dt(BF16, g, want) == 0, (algo, "streaming", r)
+    ctx.close()
