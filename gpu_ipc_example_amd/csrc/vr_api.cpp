@@ -360,17 +360,30 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     // From 64 MiB of output on: a one-trip grid (one tile per work-group).  The
     // hardware starts work-groups in index order, so the launch sweeps every stream
     // front to back with all CUs close together, where the work-groups of a
-    // persistent grid drift apart: 9 to 20 % faster on inputs no cache holds
-    // (4 x 8 MiB: 33.4 -> 30.5 us, 4 x 32 MiB: 126 -> 108 us, 2 x 64 MiB: 73 -> 66 us),
-    // as fast or faster when the inputs are cache-resident, slower only for
-    // launch-bound sizes.  From four ranks on, two sources are worked on at a time
-    // (half of the XCDs share a source's slice) rather than every XCD staying with one
-    // source: another 2-5 % (4 x 8 MiB 30.0 us, 8 x 4 MiB 53.5 -> 51.4 us); the largest
-    // eight-rank shapes do best with four work-groups per CU (8 x 16 MiB: 193.6 us).
+    // persistent grid drift apart: 9 to 20 % faster on inputs no cache holds, as fast
+    // or faster when the inputs are cache-resident, slower only for launch-bound sizes.
+    // With 48 / N waves per CU or a few more (the stores in flight per CU are what
+    // counts: a wave issues N of them per load) and the sources worked on one at a
+    // time, or two for the smaller eight-rank shapes, another 2 to 12 %.  Cold sets,
+    // HIP events, persistent grid -> uncapped one-trip grid -> this:
+    //   4 x 8 MiB 33.4 -> 30.5 -> 29.4 us    4 x 32 MiB 126 -> 108 -> 102.9 us
+    //   8 x 4 MiB 62.1 -> 52.7 -> 50.5 us    8 x 16 MiB 233 -> 192.5 -> 189.1 us
+    //   2 x 16 MiB 20.2 -> 19.2 -> 18.4 us   2 x 64 MiB 73.2 -> 66.3 -> 64.2 us
     if (write_bytes >= ((size_t)64 << 20)) {
       t.oneshot = 1;
-      if (ctx->nranks >= 4) t.deal = 2;
-      if (ctx->nranks == 8 && write_bytes >= ((size_t)512 << 20)) t.wgs_per_cu = 4;
+      t.deal = 1;
+      switch (ctx->nranks) {
+        case 2:
+          t.block = 512, t.wgs_per_cu = 3;
+          break;
+        case 4:
+          t.block = 128, t.wgs_per_cu = 8;
+          break;
+        default:  // 8
+          t.block = 128, t.wgs_per_cu = 6;
+          if (write_bytes < ((size_t)512 << 20)) t.deal = 2;
+          break;
+      }
     }
   } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) < kMall) {
     // "small" family at the sizes it is meant for: every lane makes one trip;

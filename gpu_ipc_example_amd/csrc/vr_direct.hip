@@ -74,8 +74,7 @@ __device__ __forceinline__ void st(__amdgpu_buffer_rsrc_t r, uint32_t off, V v) 
     __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, off, 0, AUX);
 }
 
-// Rank whose input is the k-th operand of the chain for the chunk owned by
-// `owner`, and the chunk index itself.
+// The chunk a protocol owner reduces.
 template <int N, int ORDER>
 __device__ __forceinline__ int chunk_of_owner(int owner) {
   // (The no-add yardstick stands beside the bisect all-reduce, so it deals the
@@ -86,18 +85,53 @@ __device__ __forceinline__ int chunk_of_owner(int owner) {
     return owner;
 }
 
+// t[k] = t[(k + a) % M] for 0 <= a < M, M a power of two: log2(M) rounds of scalar
+// selects, no memory access.
+template <int M, typename T>
+__device__ __forceinline__ void rotate_left(T (&t)[M], int a) {
+#pragma unroll
+  for (int s = 1; s < M; s <<= 1) {
+    const bool bit = (a & s) != 0;
+    T u[M];
+#pragma unroll
+    for (int k = 0; k < M; ++k) u[k] = bit ? t[(k + s) % M] : t[k];
+#pragma unroll
+    for (int k = 0; k < M; ++k) t[k] = u[k];
+  }
+}
+
+// op[k] = the input that is the k-th operand of the chain for the chunk owned by
+// `owner`.  All N pointers are fetched with static indices (one scalar load of the
+// whole table) and permuted in registers: a table lookup per operand would be N
+// dependent scalar loads at the head of every work-group.
 template <int N, int ORDER>
-__device__ __forceinline__ int operand_rank(int owner, int k) {
+__device__ __forceinline__ void select_operands(const PtrTable &in, int owner, const char *(&op)[N]) {
   if constexpr (ORDER == ORDER_COPY) {
-    return k;
+#pragma unroll
+    for (int k = 0; k < N; ++k) op[k] = static_cast<const char *>(in.p[k]);
   } else if constexpr (ORDER == ORDER_ROTATED) {
-    return (owner + k) % N;                       // own chunk first, then rank+1, rank+2, ...
+    // own chunk first, then rank+1, rank+2, ...
+#pragma unroll
+    for (int k = 0; k < N; ++k) op[k] = static_cast<const char *>(in.p[k]);
+    rotate_left<N>(op, owner);
   } else {
+    // pair sums in the order l, l+1, ... (mod N/2); inside a pair the rank of the
+    // owner's parity supplies its own data (even k) and its partner the message (odd k)
     constexpr int B = N / 2;
     const int h = owner & 1, l = owner >> 1;
-    const int j = (l + (k >> 1)) % B;             // pair index walks l, l+1, ...
-    const int self = 2 * j + h;                   // the same-parity rank that formed pair sum j
-    return (k & 1) ? (self ^ 1) : self;           // k even: its own data; k odd: its pair's message
+    const char *ev[B], *od[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      ev[j] = static_cast<const char *>(in.p[2 * j]);
+      od[j] = static_cast<const char *>(in.p[2 * j + 1]);
+    }
+    rotate_left<B>(ev, l);
+    rotate_left<B>(od, l);
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      op[2 * j] = h ? od[j] : ev[j];      // k even: the same-parity rank that formed pair sum j
+      op[2 * j + 1] = h ? ev[j] : od[j];  // k odd: its pair's message
+    }
   }
 }
 
@@ -142,21 +176,23 @@ template <int N, int ORDER, int DT, typename V, int UNROLL, int LD_AUX, int ST_A
 __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable out,
                                                            size_t chunk_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank, uint32_t deal) {
-  // `deal` chunks are worked on at a time: the first deal * blocks_per_rank work-groups
-  // belong to the first `deal` owners, round robin, and so on.  deal = N: work-group b
+                                                           uint32_t blocks_per_rank, uint32_t deal_log2) {
+  // 2^deal_log2 chunks ("deal") are worked on at a time: row y of the grid, deal *
+  // blocks_per_rank work-groups, belongs to owners y * deal ... y * deal + deal - 1,
+  // round robin (rows are dispatched one after the other).  deal = N: work-group b
   // serves owner b % N throughout (with 8 ranks every XCD its own chunk); deal = 1: all
   // work-groups, and with them all XCDs, sweep one chunk after the other.
-  const uint32_t per = deal * blocks_per_rank;
-  const uint32_t part = blockIdx.x / per, rem = blockIdx.x % per;
-  const int owner = owner_of_group<N, ORDER>((int)(part * deal + rem % deal));
-  const uint32_t jblock = rem / deal;
+  const uint32_t deal = 1u << deal_log2;
+  const int owner = owner_of_group<N, ORDER>((int)(blockIdx.y * deal + (blockIdx.x & (deal - 1))));
+  const uint32_t jblock = blockIdx.x >> deal_log2;
   const size_t base = (size_t)chunk_of_owner<N, ORDER>(owner) * chunk_pitch + seg_off;
 
+  const char *op[N];
+  select_operands<N, ORDER>(in, owner, op);
   __amdgpu_buffer_rsrc_t src[N], dst[N];
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    src[k] = make_rsrc(static_cast<const char *>(in.p[operand_rank<N, ORDER>(owner, k)]) + base, seg_bytes);
+    src[k] = make_rsrc(op[k] + base, seg_bytes);
     dst[k] = make_rsrc(static_cast<char *>(out.p[k]) + base, seg_bytes);
   }
   const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
@@ -169,6 +205,10 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
       for (int k = 0; k < N; ++k) x[u][k] = ld<V, LD_AUX>(src[k], t + u * row + lane);
+    // Every load of the trip is issued before the first add waits for one: left to
+    // itself the scheduler may hold a load back behind the adds of earlier operands,
+    // which puts a whole memory latency into the trip (measured: +4 us on 83).
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       if constexpr (ORDER == ORDER_COPY) {
@@ -190,25 +230,25 @@ template <int N, typename V, int UNROLL, int LD_AUX, int ST_AUX>
 __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable out,
                                                            size_t slice_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank, uint32_t deal) {
-  // `deal` source slices are worked on at a time (see k_direct_allreduce): deal = N gives
-  // work-group b to source b % N throughout, deal = 1 lets all work-groups sweep one
-  // source's slice after the other.
-  const uint32_t per = deal * blocks_per_rank;
-  const uint32_t part = blockIdx.x / per, rem = blockIdx.x % per;
-  const int p = (int)(part * deal + rem % deal);
-  const uint32_t jblock = rem / deal;
+                                                           uint32_t blocks_per_rank, uint32_t deal_log2) {
+  // 2^deal_log2 source slices are worked on at a time (see k_direct_allreduce): deal = N
+  // gives work-group b to source b % N throughout, deal = 1 lets all work-groups sweep
+  // one source's slice after the other.
+  const uint32_t deal = 1u << deal_log2;
+  const int p = (int)(blockIdx.y * deal + (blockIdx.x & (deal - 1)));
+  const uint32_t jblock = blockIdx.x >> deal_log2;
   const char *src_ptr = static_cast<const char *>(in.p[p]) + seg_off;
   const __amdgpu_buffer_rsrc_t src = make_rsrc(src_ptr, seg_bytes);
   __amdgpu_buffer_rsrc_t dst[N];
-  bool skip[N];
 #pragma unroll
   for (int r = 0; r < N; ++r) {
     char *d = static_cast<char *>(out.p[r]) + (size_t)p * slice_pitch + seg_off;
     // The reference skips the store when a rank's input already is its own
-    // output slot (sequential_transmit.hpp:496-497).
-    skip[r] = d == src_ptr;
-    dst[r] = make_rsrc(d, seg_bytes);
+    // output slot (sequential_transmit.hpp:496-497).  Here such a destination gets
+    // a resource of length zero, so the hardware drops its stores: no branch sits
+    // between the N stores of a trip (with branches there, launches with few waves
+    // per CU ran up to 20 % slower).
+    dst[r] = make_rsrc(d, d == src_ptr ? 0u : seg_bytes);
   }
   const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
   const uint32_t row = blockDim.x * (uint32_t)sizeof(V);
@@ -221,8 +261,7 @@ __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-      for (int r = 0; r < N; ++r)
-        if (!skip[r]) st<V, ST_AUX>(dst[r], t + u * row + lane, x[u]);
+      for (int r = 0; r < N; ++r) st<V, ST_AUX>(dst[r], t + u * row + lane, x[u]);
   }
 }
 
@@ -345,11 +384,12 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   // chunks dealt at a time: a divisor of N, N itself unless the launch says otherwise
-  uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
+  const uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
+  const uint32_t deal_log2 = (uint32_t)__builtin_ctz(deal);   // N is a power of two, so are its divisors
   for (size_t off = 0; off < chunk_bytes; off += seg_max) {
     const size_t seg = chunk_bytes - off < seg_max ? chunk_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
-    const dim3 grid(bpr * N), block(t.block);
+    const dim3 grid(bpr * deal, N / deal), block(t.block);
     // kernel-attached profiling events: start on the first segment, stop on the last
     hipEvent_t ev0 = off == 0 ? tl_kernel_events.start : nullptr;
     hipEvent_t ev1 = off + seg >= chunk_bytes ? tl_kernel_events.stop : nullptr;
@@ -357,9 +397,9 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
       auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
@@ -431,19 +471,20 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   const uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
+  const uint32_t deal_log2 = (uint32_t)__builtin_ctz(deal);
   for (size_t off = 0; off < slice_bytes; off += seg_max) {
     const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);
-    const dim3 grid(bpr * N), block(t.block);
+    const dim3 grid(bpr * deal, N / deal), block(t.block);
     hipEvent_t ev0 = off == 0 ? tl_kernel_events.start : nullptr;
     hipEvent_t ev1 = off + seg >= slice_bytes ? tl_kernel_events.stop : nullptr;
     hipError_t e = with_policy(t, [&](auto ld_aux, auto st_aux) {
       auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
