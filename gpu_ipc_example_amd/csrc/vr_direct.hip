@@ -176,7 +176,8 @@ template <int N, int ORDER, int DT, typename V, int UNROLL, int LD_AUX, int ST_A
 __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable out,
                                                            size_t chunk_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank, uint32_t deal_log2) {
+                                                           uint32_t blocks_per_rank, uint32_t deal_log2,
+                                                           uint32_t row) {
   // 2^deal_log2 chunks ("deal") are worked on at a time: row y of the grid, deal *
   // blocks_per_rank work-groups, belongs to owners y * deal ... y * deal + deal - 1,
   // round robin (rows are dispatched one after the other).  deal = N: work-group b
@@ -196,10 +197,14 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
     dst[k] = make_rsrc(static_cast<char *>(out.p[k]) + base, seg_bytes);
   }
   const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
-  const uint32_t row = blockDim.x * (uint32_t)sizeof(V);       // bytes one unroll step spans
+  // `row` = bytes one unroll step spans, blockDim.x * sizeof(V): an argument, so that it
+  // arrives with the others instead of through a separate load of the launch's dimensions
   const uint32_t tile = row * UNROLL;
   const uint32_t stride = tile * blocks_per_rank;
-  for (uint32_t t = jblock * tile; t < seg_bytes; t += stride) {
+  // Every work-group has a first tile (the host launches at most one work-group per tile),
+  // so the loop tests at its end and nothing separates the kernel's argument loads.
+  uint32_t t = jblock * tile;
+  do {
     V x[UNROLL][N];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
@@ -221,7 +226,8 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
         for (int k = 0; k < N; ++k) st<V, ST_AUX>(dst[k], t + u * row + lane, acc);
       }
     }
-  }
+    t += stride;
+  } while (t < seg_bytes);
 }
 
 // All-gather: the groups of rank p read p's slice once and store it into slot p
@@ -230,14 +236,20 @@ template <int N, typename V, int UNROLL, int LD_AUX, int ST_AUX>
 __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable out,
                                                            size_t slice_pitch, size_t seg_off,
                                                            uint32_t seg_bytes,
-                                                           uint32_t blocks_per_rank, uint32_t deal_log2) {
+                                                           uint32_t blocks_per_rank, uint32_t deal_log2,
+                                                           uint32_t row) {
   // 2^deal_log2 source slices are worked on at a time (see k_direct_allreduce): deal = N
   // gives work-group b to source b % N throughout, deal = 1 lets all work-groups sweep
   // one source's slice after the other.
   const uint32_t deal = 1u << deal_log2;
   const int p = (int)(blockIdx.y * deal + (blockIdx.x & (deal - 1)));
   const uint32_t jblock = blockIdx.x >> deal_log2;
-  const char *src_ptr = static_cast<const char *>(in.p[p]) + seg_off;
+  // the source pointer picked from the whole table with scalar selects: a look-up
+  // by p would be a second, dependent scalar load at the head of every work-group
+  uintptr_t picked = 0;
+#pragma unroll
+  for (int k = 0; k < N; ++k) picked |= p == k ? reinterpret_cast<uintptr_t>(in.p[k]) : (uintptr_t)0;
+  const char *src_ptr = reinterpret_cast<const char *>(picked) + seg_off;
   const __amdgpu_buffer_rsrc_t src = make_rsrc(src_ptr, seg_bytes);
   __amdgpu_buffer_rsrc_t dst[N];
 #pragma unroll
@@ -251,10 +263,10 @@ __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable
     dst[r] = make_rsrc(d, d == src_ptr ? 0u : seg_bytes);
   }
   const uint32_t lane = threadIdx.x * (uint32_t)sizeof(V);
-  const uint32_t row = blockDim.x * (uint32_t)sizeof(V);
   const uint32_t tile = row * UNROLL;
   const uint32_t stride = tile * blocks_per_rank;
-  for (uint32_t t = jblock * tile; t < seg_bytes; t += stride) {
+  uint32_t t = jblock * tile;   // every work-group has a first tile, as in k_direct_allreduce
+  do {
     V x[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) x[u] = ld<V, LD_AUX>(src, t + u * row + lane);
@@ -262,7 +274,8 @@ __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable
     for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
       for (int r = 0; r < N; ++r) st<V, ST_AUX>(dst[r], t + u * row + lane, x[u]);
-  }
+    t += stride;
+  } while (t < seg_bytes);
 }
 
 // Streaming yardsticks over one segment: MODE 0 copies, 1 only reads (the sum is
@@ -380,7 +393,8 @@ static hipError_t with_policy(const Tuning &t, F &&f) {
 template <int N, int ORDER, int DT, typename V, int UNROLL>
 static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
                                      const PtrTable &in, const PtrTable &out, size_t chunk_bytes) {
-  const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
+  const uint32_t row = (uint32_t)(t.block * sizeof(V));   // bytes one unroll step of a work-group spans
+  const size_t tile = (size_t)row * UNROLL;
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   // chunks dealt at a time: a divisor of N, N itself unless the launch says otherwise
@@ -397,9 +411,9 @@ static hipError_t launch_ar_segments(hipStream_t s, const DeviceInfo &dev, const
       auto kernel = k_direct_allreduce<N, ORDER, DT, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2, row);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, chunk_bytes, off, (uint32_t)seg, bpr, deal_log2, row);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
@@ -467,7 +481,8 @@ hipError_t launch_direct_allreduce(hipStream_t s, const DeviceInfo &dev, const T
 template <int N, typename V, int UNROLL>
 static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const Tuning &t,
                                      const PtrTable &in, const PtrTable &out, size_t slice_bytes) {
-  const size_t tile = (size_t)t.block * sizeof(V) * UNROLL;
+  const uint32_t row = (uint32_t)(t.block * sizeof(V));   // bytes one unroll step of a work-group spans
+  const size_t tile = (size_t)row * UNROLL;
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   const uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
@@ -482,9 +497,9 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
       auto kernel = k_direct_allgather<N, V, UNROLL, decltype(ld_aux)::value, decltype(st_aux)::value>;
       if (hipError_t a = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), dev, lds); a != hipSuccess) return a;
       if (ev0 || ev1)
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, ev0, ev1, 0, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2, row);
       else
-        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2);
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, in, out, slice_bytes, off, (uint32_t)seg, bpr, deal_log2, row);
       return hipGetLastError();
     });
     if (e != hipSuccess) return e;
