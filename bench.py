@@ -70,7 +70,7 @@ KERNEL_SAMPLE_LAUNCHES = 200
 KERNEL_SAMPLE_MIN_PAIRS = 20
 # p50 kernel execution time of cfg2 in a rocprofv3 kernel trace (microseconds), and the
 # summary under profiles/ that states it; printed beside the in-process figures.
-CFG2_KERNEL_TRACE = (4.52, "direct_allreduce_small_8x1MiB_kernel_trace.md")
+CFG2_KERNEL_TRACE = (4.20, "direct_allreduce_small_8x1MiB_kernel_trace.md")
 
 # --transport: how the virtual ranks exchange data (0 = the protocol's default).
 TRANSPORT = 0
