@@ -265,6 +265,7 @@ static int *tuning_field(vr_ctx *ctx, const char *key) {
   if (!strcmp(key, "f16_wide")) return &ctx->tune.f16_wide;
   if (!strcmp(key, "wgs_per_cu")) return &ctx->tune.wgs_per_cu;
   if (!strcmp(key, "deal")) return &ctx->tune.deal;
+  if (!strcmp(key, "run")) return &ctx->tune.run;
   if (!strcmp(key, "wire_fenced")) return &ctx->tune.wire_fenced;
   if (!strcmp(key, "wire_cooperative")) return &ctx->tune.wire_cooperative;
   if (!strcmp(key, "wire_blocks_per_cu")) return &ctx->tune.wire_blocks_per_cu;
@@ -300,6 +301,8 @@ extern "C" int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value) {
       return fail(VR_ERR_INVALID, "wgs_per_cu must be in [0,12] (0 = no cap)");
     if (!strcmp(key, "deal") && (value < 0 || value > ctx->nranks || (value && ctx->nranks % value)))
       return fail(VR_ERR_INVALID, "deal must be 0 or a divisor of the rank count");
+    if (!strcmp(key, "run") && (value < 0 || value > 256 || (value & (value - 1))))
+      return fail(VR_ERR_INVALID, "run must be 0 or a power of two up to 256");
     if (!strcmp(key, "wire_ahead") && (value < 1 || value > kWireMaxSlots - 2))
       return fail(VR_ERR_INVALID, "wire_ahead must be in [1,6]");
     if (!strcmp(key, "wire_blocks_per_cu")) {
@@ -364,25 +367,37 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     // or faster when the inputs are cache-resident, slower only for launch-bound sizes.
     // With 48 / N waves per CU or a few more (the stores in flight per CU are what
     // counts: a wave issues N of them per load) and the sources worked on one at a
-    // time, or two for the smaller eight-rank shapes, another 2 to 12 %.  Cold sets,
-    // HIP events, persistent grid -> uncapped one-trip grid -> this:
+    // time, another 2 to 12 %.  Cold sets, HIP events, persistent grid -> uncapped
+    // one-trip grid -> capped:
     //   4 x 8 MiB 33.4 -> 30.5 -> 29.4 us    4 x 32 MiB 126 -> 108 -> 102.9 us
     //   8 x 4 MiB 62.1 -> 52.7 -> 50.5 us    8 x 16 MiB 233 -> 192.5 -> 189.1 us
     //   2 x 16 MiB 20.2 -> 19.2 -> 18.4 us   2 x 64 MiB 73.2 -> 66.3 -> 64.2 us
     if (write_bytes >= ((size_t)64 << 20)) {
       t.oneshot = 1;
       t.deal = 1;
+      const size_t slice = read_bytes / (size_t)ctx->nranks;
       switch (ctx->nranks) {
         case 2:
           t.block = 512, t.wgs_per_cu = 3;
           break;
         case 4:
-          t.block = 128, t.wgs_per_cu = 8;
+          t.block = 256, t.wgs_per_cu = 4;
           break;
         default:  // 8
-          t.block = 128, t.wgs_per_cu = 6;
-          if (write_bytes < ((size_t)512 << 20)) t.deal = 2;
+          if (write_bytes < ((size_t)512 << 20)) t.block = 256, t.wgs_per_cu = 3;
+          else t.block = 128, t.wgs_per_cu = 6;
           break;
+      }
+      // Up to 32 MiB of inputs in all: every XCD takes one contiguous eighth of a slice
+      // (runs of tiles / 8 consecutive tiles) instead of every eighth tile.  Alternating
+      // runs on one box, without -> with: 4 x 8 MiB 29.8 -> 28.4 us, 4 x 4 MiB 17.2 -> 15.8,
+      // 8 x 4 MiB 55.5 -> 50.6, 8 x 2 MiB 30.1 -> 27.0, 8 x 3 MiB 42.1 -> 40.5.  Longer slices gain
+      // nothing from runs (4 x 32 MiB) or lose (8 x 8 MiB +5 %, 8 x 16 MiB +9 %).
+      if (ctx->nranks >= 4 && read_bytes <= ((size_t)32 << 20)) {
+        const size_t tiles = slice / ((size_t)t.block * 16);
+        int run = 1;
+        while ((size_t)run * 2 * 8 <= tiles && run < 256) run *= 2;
+        t.run = run;
       }
     }
   } else if (a->latency_tuned && (in_place ? read_bytes : read_bytes + write_bytes) < kMall) {
@@ -479,6 +494,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   if (o.f16_wide != -1) t.f16_wide = o.f16_wide;
   if (o.wgs_per_cu != -1) t.wgs_per_cu = o.wgs_per_cu;
   if (o.deal != -1) t.deal = o.deal;
+  if (o.run != -1) t.run = o.run;
   return t;
 }
 
@@ -587,6 +603,7 @@ static int apply_user_grid(const vr_ctx *ctx, uint32_t groups, uint32_t subgroup
   t->oneshot = 0;
   t->wgs_per_cu = 0;
   t->deal = 0;
+  t->run = 0;
   t->force_blocks_per_rank = (uint32_t)div_up(groups, (size_t)ctx->nranks);
   const uint64_t w = (uint64_t)groups * subgroups;
   *wires = w > 0xffffffffull ? 0xffffffffu : (uint32_t)w;

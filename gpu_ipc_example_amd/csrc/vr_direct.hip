@@ -241,9 +241,18 @@ __global__ __launch_bounds__(1024) void k_direct_allgather(PtrTable in, PtrTable
   // 2^deal_log2 source slices are worked on at a time (see k_direct_allreduce): deal = N
   // gives work-group b to source b % N throughout, deal = 1 lets all work-groups sweep
   // one source's slice after the other.
+  const uint32_t run_log2 = deal_log2 >> 8;   // second byte: tiles per XCD run (see below)
+  deal_log2 &= 0xff;
   const uint32_t deal = 1u << deal_log2;
   const int p = (int)(blockIdx.y * deal + (blockIdx.x & (deal - 1)));
-  const uint32_t jblock = blockIdx.x >> deal_log2;
+  uint32_t jblock = blockIdx.x >> deal_log2;
+  // Consecutive work-groups run on consecutive XCDs, so XCD k gets every eighth tile.  With
+  // runs, the work-groups of each group of 8 * run are permuted so that XCD k gets `run`
+  // consecutive tiles (the ragged last group of a slice stays as it is).
+  if (run_log2) {
+    const uint32_t group = 8u << run_log2, first = jblock & ~(group - 1), r = jblock & (group - 1);
+    if (first + group <= blocks_per_rank) jblock = first + ((r & 7u) << run_log2) + (r >> 3);
+  }
   // the source pointer picked from the whole table with scalar selects: a look-up
   // by p would be a second, dependent scalar load at the head of every work-group
   uintptr_t picked = 0;
@@ -486,7 +495,9 @@ static hipError_t launch_ag_segments(hipStream_t s, const DeviceInfo &dev, const
   const size_t seg_max = segment_of(t);
   const uint32_t lds = lds_cap_bytes(dev, t.wgs_per_cu);
   const uint32_t deal = (t.deal > 0 && t.deal <= N && N % t.deal == 0) ? (uint32_t)t.deal : (uint32_t)N;
-  const uint32_t deal_log2 = (uint32_t)__builtin_ctz(deal);
+  uint32_t deal_log2 = (uint32_t)__builtin_ctz(deal);
+  // tiles per XCD run: only where a row of the grid is one source's slice and a one-trip launch
+  if (t.run > 1 && deal == 1 && t.oneshot) deal_log2 |= (uint32_t)__builtin_ctz((unsigned)t.run) << 8;
   for (size_t off = 0; off < slice_bytes; off += seg_max) {
     const size_t seg = slice_bytes - off < seg_max ? slice_bytes - off : seg_max;
     const uint32_t bpr = blocks_per_rank_for(dev, t, N, seg, tile);

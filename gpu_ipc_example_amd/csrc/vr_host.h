@@ -58,7 +58,7 @@ const AlgoInfo *algo_info(int algo);
 // User overrides of the launch heuristics; -1 = let the library decide.
 struct TuningOverrides {
   int block = -1, waves_per_cu = -1, unroll = -1, nt_load = -1, nt_store = -1, oneshot = -1;
-  int segment_kib = -1, f16_wide = -1, wgs_per_cu = -1, deal = -1;
+  int segment_kib = -1, f16_wide = -1, wgs_per_cu = -1, deal = -1, run = -1;
   int wire_fenced = -1, wire_cooperative = -1, wire_blocks_per_cu = -1, wire_ahead = -1, wire_msg16 = -1;
   int wire_stream_io = -1;
 };

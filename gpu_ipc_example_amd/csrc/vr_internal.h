@@ -44,6 +44,8 @@ struct Tuning {
   uint32_t force_blocks_per_rank = 0;  // non-zero: use exactly this many blocks per rank
   int deal = 0;           // chunks the work-groups of an all-reduce work on at a time (a divisor of the rank
                           // count; 0 = all of them: work-group b serves owner b % N throughout)
+  int run = 0;            // all-gather, one source at a time: each XCD takes runs of this many consecutive
+                          // tiles (a power of two) instead of every eighth tile; 0 or 1 = no permutation
   int wgs_per_cu = 0;     // non-zero: at most this many work-groups of the launch share a CU (the launch
                           // asks for dynamic LDS it never touches, so that no more fit); for one-trip grids,
                           // whose residency the grid size does not bound

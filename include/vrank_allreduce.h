@@ -321,6 +321,9 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * "deal" (chunks the work-groups of an all-reduce work on at a time: a divisor
  * of the rank count, 0 = all of them, i.e. work-group b serves owner b % N
  * throughout; 1 = all compute units sweep one chunk after the other),
+ * "run" (all-gather, one-trip grid, one source at a time: every XCD takes runs of
+ * this many consecutive tiles, a power of two up to 256, instead of every eighth
+ * tile; 0 = no permutation),
  * "f16_wide" (1 = binary16 adds computed through
  * binary32 and rounded back after every add: the same bits, a longer ALU section),
  * "segment_kib" (KiB of a chunk one launch

@@ -524,6 +524,24 @@ def test_allgather_one_trip_sizes(ctxs, oracle):
             got = run_allgather(ctxs[nranks], "allgather_simple", ins, alias)
             for r in range(nranks):
                 assert (got[r] == want).all(), (nranks, r, alias)
+    # Runs of consecutive tiles per XCD: forced on a slice whose tile count is no multiple of
+    # the group of 8 * run work-groups (the ragged last group keeps its order) and on one
+    # shorter than a group.
+    ctx = ctxs[4]
+    for algo, n in (("allgather_simple", 4 * 1024 * 37 + 8), ("allgather_small", 4 * 1024 * 37 + 24),
+                    ("allgather_simple", 1024), ("allgather_simple", 2048 * 8 * 5)):
+        ins = H.make_inputs(oracle, 4, n, 9500, DIST_UNIFORM, -2.0, 2.0)
+        want = oracle.allgather(ins)
+        for block, cap, run in ((64, 4, 2), (256, 4, 8), (128, 0, 256), (64, 8, 16)):
+            ctx.set_tuning(oneshot=1, block=block, unroll=1, wgs_per_cu=cap, deal=1, run=run)
+            for alias in (False, True):
+                got = run_allgather(ctx, algo, ins, alias)
+                for r in range(4):
+                    assert (got[r] == want).all(), (n, block, cap, run, r, alias)
+    ctx.set_tuning(oneshot=-1, block=-1, unroll=-1, wgs_per_cu=-1, deal=-1, run=-1)
+    for bad in (3, 512, -2):
+        with pytest.raises(vr.VRError):
+            ctx.set_tuning(run=bad)
 
 
 def test_nothing_is_written_past_the_end(ctxs, oracle):
