@@ -360,7 +360,9 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     t.waves_per_cu = 32;
     t.nt_load = 0;
     t.nt_store = 2;
-    // From 64 MiB of output on: a one-trip grid (one tile per work-group).  The
+    // From 32 MiB of output on (below, launches are latency-bound and the two grids
+    // measure alike; at 32 and 48 MiB the capped one-trip launch is 3 to 17 % faster, on
+    // cache-resident and on cold inputs): a one-trip grid (one tile per work-group).  The
     // hardware starts work-groups in index order, so the launch sweeps every stream
     // front to back with all CUs close together, where the work-groups of a
     // persistent grid drift apart: 9 to 20 % faster on inputs no cache holds, as fast
@@ -372,7 +374,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     //   4 x 8 MiB 33.4 -> 30.5 -> 29.4 us    4 x 32 MiB 126 -> 108 -> 102.9 us
     //   8 x 4 MiB 62.1 -> 52.7 -> 50.5 us    8 x 16 MiB 233 -> 192.5 -> 189.1 us
     //   2 x 16 MiB 20.2 -> 19.2 -> 18.4 us   2 x 64 MiB 73.2 -> 66.3 -> 64.2 us
-    if (write_bytes >= ((size_t)64 << 20)) {
+    if (write_bytes >= ((size_t)32 << 20)) {
       t.oneshot = 1;
       t.deal = 1;
       const size_t slice = read_bytes / (size_t)ctx->nranks;
