@@ -449,7 +449,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // One-trip grids: every work-group handles one tile and ends; the hardware starts
       // work-groups in index order, so the launch sweeps the buffers front to back with
       // all CUs close together, where the work-groups of a persistent grid drift apart.
-      // Small work-groups (one wave) with a residency cap of 4 to 10 per CU keep 32 to
+      // Small work-groups (one wave) with a residency cap of 4 to 8 per CU keep 32 to
       // 64 KiB of loads per CU in flight.  `deal` says how many chunks are worked on at a
       // time, i.e. how many XCDs share a chunk (with eight ranks: deal 8 = every XCD its
       // own chunk, deal 1 = all CUs sweep one chunk after the other, which is what lets
@@ -458,7 +458,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // Measured on cold sets against the persistent grid it replaces (fractions of the
       // HBM peak, HIP events):
       //   2 ranks  0.78 -> 0.82-0.85 (128, 256 MiB per rank)
-      //   4 ranks  0.74-0.78 -> 0.82 (64 MiB), 0.75-0.79 -> 0.83 (128 MiB), 0.71 -> 0.82 (256 MiB)
+      //   4 ranks  0.74-0.78 -> 0.82 (64 MiB), 0.75-0.79 -> 0.84 (128 MiB), 0.71 -> 0.84 (256 MiB)
       //   8 ranks  0.72-0.75 -> 0.805 (32 MiB), 0.71 -> 0.79 (40, 48 MiB), 0.73 -> 0.82 (64 MiB),
       //            0.69 -> 0.81 (96 MiB), 0.72-0.74 -> 0.82 (128 MiB), 0.68-0.75 -> 0.81 (256 MiB),
       //            0.69 -> 0.78 (512 MiB)
@@ -472,8 +472,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
           t.block = 512, t.wgs_per_cu = 2;
           break;
         case 4:
-          if (chunk < 64 * MiB) t.block = 64, t.wgs_per_cu = 10, t.deal = chunk < 32 * MiB ? 2 : 1;
-          else t.block = 256, t.wgs_per_cu = 2, t.deal = 1;
+          t.block = 64, t.wgs_per_cu = 8, t.deal = 1;
           break;
         case 8:
           t.block = 64, t.deal = 1;
