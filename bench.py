@@ -201,6 +201,34 @@ def memory_clock():
     return found or None
 
 
+def device_state():
+    """Clock levels in use, power and temperatures as sysfs shows them right after the timed
+    region: boxes of one pool differ by a few per cent in every kernel, and this is what
+    can be read about why."""
+    import glob
+    found = {}
+    for dev in sorted(glob.glob("/sys/class/drm/card*/device")):
+        st = {}
+        for clk in ("sclk", "mclk", "fclk", "socclk"):
+            try:
+                cur = [l.strip().rstrip(" *") for l in open("%s/pp_dpm_%s" % (dev, clk)) if l.strip().endswith("*")]
+            except OSError:
+                continue
+            if cur:
+                st[clk] = cur[0].split(":", 1)[-1].strip()
+        for hw in glob.glob(dev + "/hwmon/hwmon*"):
+            for key, fname, scale in (("power_cap_W", "power1_cap", 1e-6), ("power_W", "power1_average", 1e-6),
+                                      ("power_W", "power1_input", 1e-6), ("temp_edge_C", "temp1_input", 1e-3),
+                                      ("temp_junction_C", "temp2_input", 1e-3), ("temp_memory_C", "temp3_input", 1e-3)):
+                try:
+                    st.setdefault(key, round(int(open("%s/%s" % (hw, fname)).read()) * scale, 1))
+                except (OSError, ValueError):
+                    pass
+        if st:
+            found[dev.split("/")[4]] = st
+    return found or None
+
+
 def multi_stream_copy(binding, ctx, name, sets, iters, group):
     """The all-reduce kernel itself with the adds removed (N read streams, N write
     streams, same grid, addressing and cache policies), on the same rotating
@@ -650,6 +678,7 @@ def main():
                            if len(sets) > 1 else "every step reuses one buffer set (cache-warm)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "memory_clock": memory_clock(),
+        "device_state": device_state(),
         "bit_exact_vs_oracle": None,
         "roofline": roofline,
     }
