@@ -58,3 +58,34 @@ def test_random_cases(oracle, seed):
                 assert (a == b).all(), what
     for c in ctxs.values():
         c.close()
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_allgather_cases(oracle, seed):
+    """The all-gather under random launch shapes of the direct transport: one-trip or
+    persistent grid, block size, residency cap, sources dealt at a time, tile runs per
+    XCD, vectors per lane, own slot aliased or not."""
+    from tests.test_gpu_direct import run_allgather
+    from tests.oracle_lib import DIST_UNIFORM
+    rng = random.Random(5000 + seed)
+    ctxs = {n: vr.VirtualRanks(n) for n in (2, 4, 8)}
+    for case in range(30):
+        nranks = rng.choice((2, 4, 8))
+        algo = rng.choice(("allgather_small", "allgather_simple"))
+        n = 8 * rng.choice((1, 3, 17, 128, 129, 1000, 4099, 65536 // 8, rng.randrange(1, 60000)))
+        alias = rng.random() < 0.4
+        knobs = dict(oneshot=rng.choice((-1, 0, 1, 1)), block=rng.choice((-1, 64, 128, 256, 512, 1024)),
+                     wgs_per_cu=rng.choice((-1, 0, 1, 3, 8, 12)), deal=rng.choice((-1, 0, 1, 1, 2, nranks)),
+                     run=rng.choice((-1, 0, 1, 2, 8, 64, 256)), unroll=rng.choice((-1, 1, 2)),
+                     segment_kib=rng.choice((-1, -1, 4, 64)), nt_load=rng.choice((-1, 0, 1)),
+                     nt_store=rng.choice((-1, 0, 1, 2)))
+        ctxs[nranks].set_tuning(**knobs)
+        ins = H.make_inputs(oracle, nranks, n, 20_000 * seed + 41 * case, DIST_UNIFORM, -2.0, 2.0)
+        what = "seed=%d case=%d %s N=%d n=%d alias=%s knobs=%s" % (seed, case, algo, nranks, n, alias, knobs)
+        print(what, flush=True)
+        want = oracle.allgather(ins)
+        got = run_allgather(ctxs[nranks], algo, ins, alias)
+        for r in range(nranks):
+            assert (got[r] == want).all(), (what, r)
+    for c in ctxs.values():
+        c.close()
