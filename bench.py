@@ -201,6 +201,17 @@ def memory_clock():
     return found or None
 
 
+def launch_plan(binding, algo, n, ne, args):
+    """The launch the library picks for the timed workload on the direct transport
+    (vr_direct_launch_plan), with the --tune overrides of this run beside it."""
+    if args.transport not in ("default", "direct") or algo == "parallel":
+        return None
+    plan = binding.direct_launch_plan(algo, n, ne, bool(args.inplace))
+    if args.tune:
+        plan["overridden_by_--tune"] = list(args.tune)
+    return plan
+
+
 def device_state():
     """Clock levels in use, power and temperatures as sysfs shows them right after the timed
     region: boxes of one pool differ by a few per cent in every kernel, and this is what
@@ -497,7 +508,8 @@ def allgather_block(vr, binding, want_check, gpu_results):
     gb = B / (float(kms.mean()) * 1e-3) / 1e9
     out = {"workload": describe(name), "GBps": round(gb, 1), "frac_of_hbm_peak": round(gb / HBM_PEAK_GBPS, 4),
            "algorithmic_bytes_per_step": B, "traffic": measured_traffic(name, "default"),
-           "buffer_sets_rotated": len(s4), "bit_exact_vs_oracle": None}
+           "buffer_sets_rotated": len(s4), "bit_exact_vs_oracle": None,
+           "launch": binding.direct_launch_plan(WORKLOADS[name][1], WORKLOADS[name][0], WORKLOADS[name][2], False)}
     out.update(stats)
     time_kernels(binding, c4, name, s4[:4], 8)
     warm, wstats = kernel_sample(binding, c4, name, s4[:4], 10)
@@ -677,6 +689,7 @@ def main():
                                len(sets), len(sets) * (B if not args.inplace else B / 2) / 2**20)
                            if len(sets) > 1 else "every step reuses one buffer set (cache-warm)"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "launch": launch_plan(binding, algo, n, ne, args),
         "memory_clock": memory_clock(),
         "device_state": device_state(),
         "bit_exact_vs_oracle": None,

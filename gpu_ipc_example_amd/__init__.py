@@ -16,6 +16,7 @@ from .binding import (  # noqa: F401
     build_library,
     check_allreduce,
     launch_geometry,
+    direct_launch_plan,
     lib,
     library_path,
     parse_nelems,

@@ -39,6 +39,11 @@ class Geometry(C.Structure):
     _fields_ = [("groups", C.c_uint32), ("subgroups", C.c_uint32), ("steps", C.c_uint32)]
 
 
+class LaunchPlan(C.Structure):
+    _fields_ = [(k, C.c_int) for k in ("one_trip", "block", "unroll", "waves_per_cu", "wgs_per_cu", "deal", "run",
+                                       "nt_load", "nt_store", "f16_wide")]
+
+
 def library_path():
     return _SO
 
@@ -97,6 +102,7 @@ def lib():
         "vr_allreduce_grid": (i, [vp, vp, i, i, vpp, vpp, sz, u32, u32, u32, u32]),
         "vr_ctx_check": (i, [vp, vp]),
         "vr_ctx_set_spin_limit": (i, [vp, C.c_uint64]),
+        "vr_direct_launch_plan": (i, [i, i, sz, i, C.POINTER(LaunchPlan)]),
         "vr_ctx_set_tuning": (i, [vp, C.c_char_p, i]),
         "vr_ctx_get_tuning": (i, [vp, C.c_char_p, C.POINTER(i)]),
         "vr_time_allreduce": (i, [vp, vp, i, i, vpp, vpp, sz, i, C.POINTER(C.c_float)]),
@@ -171,6 +177,13 @@ def launch_geometry(algo, nranks, nelems):
     g = Geometry()
     _check(lib().vr_launch_geometry(algo_id(algo), nranks, nelems, C.byref(g)))
     return g.groups, g.subgroups, g.steps
+
+
+def direct_launch_plan(algo, nranks, nelems, in_place=True):
+    """The launch the direct transport picks for this shape (a dict; no GPU needed)."""
+    p = LaunchPlan()
+    _check(lib().vr_direct_launch_plan(algo_id(algo), nranks, nelems, int(in_place), C.byref(p)))
+    return {k: getattr(p, k) for k, _ in LaunchPlan._fields_}
 
 
 DTYPE_F16, DTYPE_BF16 = 0, 1

@@ -346,8 +346,8 @@ bool ranges_partially_overlap(const void *a, const void *b, size_t bytes) {
 // the 256 MiB memory-side cache (Infinity Cache) in front of HBM.  Store policy 2
 // (streaming, written through at agent scope) is the fastest way to HBM but takes
 // the results out of the L2 a following in-place launch would read them from.
-static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes, size_t write_bytes,
-                         bool in_place) {
+static Tuning default_tuning(int nranks, const AlgoInfo *a, size_t read_bytes, size_t write_bytes,
+                             bool in_place) {
   const size_t kMall = 256ull << 20;
   Tuning t;
   t.block = 256;
@@ -377,8 +377,8 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     if (write_bytes >= ((size_t)32 << 20)) {
       t.oneshot = 1;
       t.deal = 1;
-      const size_t slice = read_bytes / (size_t)ctx->nranks;
-      switch (ctx->nranks) {
+      const size_t slice = read_bytes / (size_t)nranks;
+      switch (nranks) {
         case 2:
           t.block = 512, t.wgs_per_cu = 3;
           break;
@@ -395,7 +395,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       // runs on one box, without -> with: 4 x 8 MiB 29.8 -> 28.4 us, 4 x 4 MiB 17.2 -> 15.8,
       // 8 x 4 MiB 55.5 -> 50.6, 8 x 2 MiB 30.1 -> 27.0, 8 x 3 MiB 42.1 -> 40.5.  Longer slices gain
       // nothing from runs (4 x 32 MiB) or lose (8 x 8 MiB +5 %, 8 x 16 MiB +9 %).
-      if (ctx->nranks >= 4 && read_bytes <= ((size_t)32 << 20)) {
+      if (nranks >= 4 && read_bytes <= ((size_t)32 << 20)) {
         const size_t tiles = slice / ((size_t)t.block * 16);
         int run = 1;
         while ((size_t)run * 2 * 8 <= tiles && run < 256) run *= 2;
@@ -416,7 +416,7 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     // equal or up to 5 % faster at every size from 2 to 32 MiB per rank, in place and
     // out of place, and 3 % faster when an in-place 256 MiB set turns out not to be
     // resident after all.
-    const int cached_waves = ctx->nranks == 8 ? 4 : 8;
+    const int cached_waves = nranks == 8 ? 4 : 8;
     // (A footprint of exactly the cache's size counts as streaming: nothing else may have
     // touched memory for it to be resident, and the streaming launch takes 82 us on eight
     // 32 MiB buffers in place whether they are resident or not, where the cached policy
@@ -439,13 +439,13 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
     } else {
       // Pure streaming.  DRAM runs best with about 32 loads per CU in flight:
       // N loads per lane times 4 waves (8 waves for two ranks).
-      t.waves_per_cu = ctx->nranks >= 4 ? 4 : 8;
+      t.waves_per_cu = nranks >= 4 ? 4 : 8;
       t.nt_load = 1;
       t.nt_store = 2;
       // Same sums, computed through binary32: the longer ALU section between a
       // trip's loads and its stores shortens the launch by 2.5 % at 8 ranks (0.5 %
       // at 4; it costs 1-2 % at 2 and 16 ranks and 8 % when the data is cache-resident).
-      t.f16_wide = ctx->nranks == 4 || ctx->nranks == 8;
+      t.f16_wide = nranks == 4 || nranks == 8;
       // One-trip grids: every work-group handles one tile and ends; the hardware starts
       // work-groups in index order, so the launch sweeps the buffers front to back with
       // all CUs close together, where the work-groups of a persistent grid drift apart.
@@ -463,11 +463,11 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       //            0.69 -> 0.81 (96 MiB), 0.72-0.74 -> 0.82 (128 MiB), 0.68-0.75 -> 0.81 (256 MiB),
       //            0.69 -> 0.78 (512 MiB)
       //   16 ranks 0.68-0.70 -> 0.75 (16 MiB), 0.72 -> 0.78 (32 MiB), 0.71 -> 0.79 (64 MiB)
-      const size_t chunk = read_bytes / ((size_t)ctx->nranks * ctx->nranks);
+      const size_t chunk = read_bytes / ((size_t)nranks * nranks);
       const size_t MiB = (size_t)1 << 20;
       t.oneshot = 1;
       t.unroll = 1;
-      switch (ctx->nranks) {
+      switch (nranks) {
         case 2:
           t.block = 512, t.wgs_per_cu = 2;
           break;
@@ -484,6 +484,13 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
       }
     }
   }
+  return t;
+}
+
+// The same with the context's overrides (vr_ctx_set_tuning) applied.
+static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes, size_t write_bytes,
+                         bool in_place) {
+  Tuning t = default_tuning(ctx->nranks, a, read_bytes, write_bytes, in_place);
   const TuningOverrides &o = ctx->tune;
   if (o.block != -1) t.block = o.block;
   if (o.waves_per_cu != -1) t.waves_per_cu = o.waves_per_cu;
@@ -499,6 +506,28 @@ static Tuning tuning_for(const vr_ctx *ctx, const AlgoInfo *a, size_t read_bytes
   return t;
 }
 
+
+extern "C" int vr_direct_launch_plan(int algo, int nranks, size_t nelems, int in_place, vr_launch_plan *out) {
+  const AlgoInfo *a = algo_info(algo);
+  if (!a) return fail(VR_ERR_ALGO, "unknown algo");
+  if (!out) return fail(VR_ERR_INVALID, "null plan");
+  if (nranks != 2 && nranks != 4 && nranks != 8 && nranks != 16) return fail(VR_ERR_TOPOLOGY, "nranks");
+  if (nelems > kMaxElems) return fail(VR_ERR_INVALID, "nelems too large");
+  const size_t in_bytes = (size_t)nranks * nelems * 2;
+  const Tuning t = a->allgather ? default_tuning(nranks, a, in_bytes, in_bytes * nranks, false)
+                                : default_tuning(nranks, a, in_bytes, in_bytes, in_place != 0);
+  out->one_trip = t.oneshot;
+  out->block = t.block;
+  out->unroll = t.unroll;
+  out->waves_per_cu = t.oneshot ? 0 : t.waves_per_cu;
+  out->wgs_per_cu = t.wgs_per_cu;
+  out->deal = t.deal > 0 ? t.deal : nranks;
+  out->run = t.run > 1 ? t.run : 1;
+  out->nt_load = t.nt_load;
+  out->nt_store = t.nt_store;
+  out->f16_wide = t.f16_wide;
+  return VR_OK;
+}
 
 namespace vr {
 int prepare_allreduce(vr_ctx *ctx, int algo, void *const bufs[], void *const outs[],

@@ -350,6 +350,24 @@ int vr_ctx_set_spin_limit(vr_ctx *ctx, uint64_t polls);
  * "wire_blocks_per_cu" (1..4 resident work-groups per CU; set it before
  * vr_ctx_reserve_wire, it sizes the scratch).
  * -1 restores the library's own choice. */
+/* The launch the direct transport gives a collective of this shape when nothing
+ * is overridden: pure host arithmetic, no device needed (nelems per rank; in_place
+ * is ignored for an all-gather).  No counterpart in the reference, whose launch
+ * shape is the user's -g / -w / -s (main.cpp:181-198). */
+typedef struct vr_launch_plan {
+  int one_trip;      /* 1: one tile per work-group, started in index order; 0: persistent grid-stride grid */
+  int block;         /* threads per work-group */
+  int unroll;        /* vectors in flight per lane and rank */
+  int waves_per_cu;  /* persistent grid: waves per compute unit; 0 for a one-trip grid */
+  int wgs_per_cu;    /* one-trip grid: residency cap in work-groups per compute unit, 0 = none */
+  int deal;          /* chunks (all-gather: sources) worked on at a time */
+  int run;           /* all-gather: consecutive tiles per XCD (1 = every eighth tile) */
+  int nt_load;       /* 0 cached, 1 streaming loads */
+  int nt_store;      /* 0 cached, 1 streaming, 2 streaming and written through at agent scope */
+  int f16_wide;      /* 1: binary16 adds computed through binary32 (same bits) */
+} vr_launch_plan;
+int vr_direct_launch_plan(int algo, int nranks, size_t nelems, int in_place, vr_launch_plan *out);
+
 int vr_ctx_set_tuning(vr_ctx *ctx, const char *key, int value);
 int vr_ctx_get_tuning(vr_ctx *ctx, const char *key, int *value);
 

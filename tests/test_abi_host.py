@@ -127,3 +127,55 @@ def test_no_device_is_a_clean_error():
     with pytest.raises(vr.VRError) as e:
         vr.VirtualRanks(8)
     assert e.value.code == "NO_DEVICE"
+
+
+def test_launch_plans_of_the_direct_transport():
+    """The launches the library picks by itself, as its documentation states them (pure host
+    arithmetic behind vr_direct_launch_plan)."""
+    MiB = 1 << 20
+    plan = vr.direct_launch_plan
+    # the headline shape: one-trip grid of one-wave work-groups, five per CU, one chunk at a time,
+    # streaming loads, streaming stores written through, adds through binary32; in place alike
+    for in_place in (False, True):
+        p = plan("bisect", 8, 16 * MiB, in_place)
+        assert (p["one_trip"], p["block"], p["unroll"], p["wgs_per_cu"], p["deal"]) == (1, 64, 1, 5, 1)
+        assert (p["nt_load"], p["nt_store"], p["f16_wide"]) == (1, 2, 1)
+    # other rank counts when streaming
+    p = plan("bisect", 4, 32 * MiB, True)
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["deal"], p["f16_wide"]) == (1, 64, 8, 1, 1)
+    p = plan("simple", 2, 64 * MiB, True)
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["f16_wide"]) == (1, 512, 2, 0)
+    assert (plan("bisect", 16, 8 * MiB, True)["deal"], plan("bisect", 16, 16 * MiB, True)["deal"]) == (2, 1)
+    assert plan("bisect", 16, 8 * MiB, True)["wgs_per_cu"] == 4
+    # eight ranks: six work-groups per CU for chunks of 16 to 32 MiB
+    assert [plan("bisect", 8, n * MiB // 2, True)["wgs_per_cu"] for n in (64, 128, 256, 512)] == [5, 6, 6, 5]
+    # everything fits the memory-side cache: persistent grid, cacheable loads, streaming stores
+    p = plan("simple", 8, 4 * MiB, True)
+    assert (p["one_trip"], p["waves_per_cu"], p["deal"], p["nt_load"], p["nt_store"], p["f16_wide"]) == (0, 4, 8, 0, 1, 0)
+    assert plan("simple", 4, 4 * MiB, True)["waves_per_cu"] == 8
+    # an in-place footprint of exactly the cache's size streams; one element less does not
+    assert plan("bisect", 8, 16 * MiB, True)["nt_load"] == 1 and plan("bisect", 8, 16 * MiB - 64, True)["nt_load"] == 0
+    # out of place: inputs about the size of the L2s -> results written through; inputs up to half
+    # the cache with a footprint beyond it -> cached loads, results streamed past them
+    assert plan("simple", 8, 2 * MiB, False)["nt_store"] == 2 and plan("simple", 8, 1 * MiB, False)["nt_store"] == 1
+    p = plan("bisect", 8, 8 * MiB, False)
+    assert (p["one_trip"], p["nt_load"], p["nt_store"]) == (0, 0, 2)
+    # the latency family: one trip per lane, everything cacheable, up to the size of the cache
+    p = plan("small", 8, MiB // 2, True)
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["nt_load"], p["nt_store"]) == (1, 256, 0, 0, 0)
+    assert plan("small", 8, 16 * MiB, True)["nt_load"] == 1
+    # all-gather: persistent below 32 MiB of output, capped one-trip launches from there on, tile
+    # runs (one contiguous eighth of a slice per XCD) up to 32 MiB of inputs
+    p = plan("allgather_simple", 4, MiB // 2, False)
+    assert (p["one_trip"], p["waves_per_cu"], p["nt_load"], p["nt_store"]) == (0, 32, 0, 2)
+    p = plan("allgather_simple", 4, 4 * MiB, False)                     # config 4
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["deal"], p["run"]) == (1, 256, 4, 1, 256)
+    p = plan("allgather_simple", 8, 2 * MiB, False)
+    assert (p["block"], p["wgs_per_cu"], p["deal"], p["run"]) == (256, 3, 1, 128)
+    p = plan("allgather_simple", 8, 8 * MiB, False)
+    assert (p["block"], p["wgs_per_cu"], p["deal"], p["run"]) == (128, 6, 1, 1)
+    p = plan("allgather_simple", 2, 8 * MiB, False)
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["run"]) == (1, 512, 3, 1)
+    assert plan("allgather_simple", 4, 16 * MiB, False)["run"] == 1
+    with pytest.raises(vr.VRError):
+        plan("bisect", 3, 1024, True)

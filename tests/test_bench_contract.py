@@ -51,7 +51,7 @@ def test_default_line_carries_the_fixed_sample_and_the_other_configurations():
                 "cfg4_allgather", "cfg5_sweep_points", "latency_1MiB_per_rank", "host_call_us",
                 "back_to_back_us_per_launch", "kernel_trace_p50_us", "same_buffers_cache_warm",
                 "hbm_ceilings", "cpu_baseline", "roofline", "inputs_cache_resident", "buffer_sets_rotated",
-                "memory_clock", "device_state"):
+                "memory_clock", "device_state", "launch"):
         assert '"%s"' % key in src, key
     us, fname = bench.CFG2_KERNEL_TRACE
     text = open(os.path.join(ROOT, "profiles", fname)).read()
