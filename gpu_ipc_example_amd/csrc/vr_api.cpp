@@ -432,6 +432,14 @@ static Tuning default_tuning(int nranks, const AlgoInfo *a, size_t read_bytes, s
       // written-through stores end them 0.3-0.5 us later; no difference beyond.
       const size_t MiB = (size_t)1 << 20;
       if (!in_place && read_bytes > 24 * MiB && read_bytes <= 40 * MiB) t.nt_store = 2;
+      // Four ranks, in place, from 96 MiB on: the one-trip grid of the streaming sizes
+      // with the cacheable policy.  A little faster than the persistent grid when the data
+      // is resident and 4 to 11 % faster when it turns out not to be (96 / 160 / 248 MiB in
+      // all, resident: 30.7 -> 30.1, 49.3 -> 48.1, 82.3 -> 79.6 us; not resident: 40.9 -> 39.2,
+      // 68.4 -> 61.1, 99.4 -> 89.2 us).  Below 80 MiB the persistent grid leads (48 MiB: 13.8
+      // against 19.4 us), at eight ranks it leads throughout, at two the two are even.
+      if (in_place && nranks == 4 && footprint >= 96 * MiB)
+        t.oneshot = 1, t.block = 64, t.wgs_per_cu = 8, t.deal = 1;
     } else if (read_bytes <= kMall / 2) {  // inputs may still be resident; stream the results past them
       t.waves_per_cu = cached_waves;
       t.nt_load = 0;

@@ -153,6 +153,11 @@ def test_launch_plans_of_the_direct_transport():
     p = plan("simple", 8, 4 * MiB, True)
     assert (p["one_trip"], p["waves_per_cu"], p["deal"], p["nt_load"], p["nt_store"], p["f16_wide"]) == (0, 4, 8, 0, 1, 0)
     assert plan("simple", 4, 4 * MiB, True)["waves_per_cu"] == 8
+    # four ranks, in place, from 96 MiB in all: the one-trip grid with the cacheable policy
+    p = plan("bisect", 4, 12 * MiB, True)
+    assert (p["one_trip"], p["block"], p["wgs_per_cu"], p["deal"], p["nt_load"], p["nt_store"]) == (1, 64, 8, 1, 0, 1)
+    assert plan("bisect", 4, 11 * MiB, True)["one_trip"] == 0 and plan("bisect", 4, 12 * MiB, False)["one_trip"] == 0
+    assert plan("bisect", 8, 6 * MiB, True)["one_trip"] == 0 and plan("simple", 2, 24 * MiB, True)["one_trip"] == 0
     # an in-place footprint of exactly the cache's size streams; one element less does not
     assert plan("bisect", 8, 16 * MiB, True)["nt_load"] == 1 and plan("bisect", 8, 16 * MiB - 64, True)["nt_load"] == 0
     # out of place: inputs about the size of the L2s -> results written through; inputs up to half
