@@ -212,8 +212,9 @@ __global__ __launch_bounds__(1024) void k_direct_allreduce(PtrTable in, PtrTable
       for (int k = 0; k < N; ++k) x[u][k] = ld<V, LD_AUX>(src[k], t + u * row + lane);
     // Every load of the trip is issued before the first add waits for one: left to
     // itself the scheduler may hold a load back behind the adds of earlier operands,
-    // which puts a whole memory latency into the trip (measured: +4 us on 83).
-    __builtin_amdgcn_sched_barrier(0);
+    // which puts a whole memory latency into the trip (measured: +4 us on 83).  (Not
+    // where a trip's loads alone fill 64 registers or more: pinned there, they spill.)
+    if constexpr (UNROLL * N * sizeof(V) <= 256) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       if constexpr (ORDER == ORDER_COPY) {
@@ -437,7 +438,8 @@ static hipError_t launch_ar_unroll(hipStream_t s, const DeviceInfo &dev, const T
   // binary32 temporaries, which leaves no room for four vectors per rank.
   const int unroll = (N >= 16) ? 1 : (t.unroll >= 4 ? 4 : (t.unroll >= 2 ? 2 : 1));
   if constexpr (N <= 8) {
-    if constexpr (DT == DT_F16)
+    // (the no-add yardstick at eight ranks would hold 128 registers of loaded data: two vectors at most)
+    if constexpr (DT == DT_F16 && !(ORDER == ORDER_COPY && N == 8))
       if (unroll == 4) return launch_ar_segments<N, ORDER, DT, V, 4>(s, dev, t, in, out, chunk_bytes);
     if (unroll >= 2) return launch_ar_segments<N, ORDER, DT, V, 2>(s, dev, t, in, out, chunk_bytes);
   }
